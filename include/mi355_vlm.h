@@ -501,6 +501,60 @@ int mi355_attn_generic_dropout_bwd(int B, int S, int Hq, int Hkv, int D, const v
                                    void* dq, int64_t lddq, void* dk, int64_t lddk, void* dv, int64_t lddv, const uint8_t* key_mask, float scale,
                                    float p, uint64_t seed, uint64_t offset, void* stream);
 
+/* ---------------------------------------------------------------------------------------------------------------------
+ * Ragged-batch serving of hybrid decoders (csrc/seqmix.hip, csrc/bgemm.hip, csrc/latent_attn.hip).  Rows are the tokens of a packed batch;
+ * sequences are described by int32 device arrays; the residual stream, norm statistics, rotary angles, decays, recurrent state and router
+ * arithmetic are fp32 whatever the activation dtype (a MI355_DT_* code per operand).
+ * ------------------------------------------------------------------------------------------------------------------- */
+/* out[t] = table[tok[t]] * scale + bigram[row], row = (prev[t] * mul_prev + tok[t] * mul_cur) mod buckets, or row `buckets` if prev[t] < 0.
+ * table / bigram bf16 (bigram may be NULL), out fp32 [tokens, width]. */
+int mi355_embed_hash_fwd(int64_t tokens, int width, int vocab, const int* tok, const int* prev, const void* table, float scale, const void* bigram,
+                         int buckets, int mul_prev, int mul_cur, float* out, void* stream);
+/* out = LayerNorm(alpha * x + sum_{p < parts} y[t * parts + p]) * w + b on fp32 rows (two-pass variance); y (dtype y_dt, row pitch ldy) may be NULL;
+ * `cast` (may be NULL) receives the same rows in dtype cast_dt. */
+int mi355_add_layernorm_fwd(int64_t tokens, int width, const float* x, float alpha, const void* y, int y_dt, int64_t ldy, int parts, const float* w,
+                            const float* b, float eps, float* out, void* cast, int cast_dt, void* stream);
+/* out[t, :n] = x[t, :n] / sqrt(mean(x[t, :n]^2) + eps) * w on strided rows. */
+int mi355_rmsnorm_rows(int64_t tokens, int n, const void* x, int x_dt, int64_t ldx, const float* w, float eps, void* out, int out_dt, int64_t ldo,
+                       void* stream);
+/* Latent key/value rows: src[t] = [rank | rot] values; cache row dst_row[t] <- [RMSNorm(first rank) * w | last rot with the pairs (2i, 2i+1), 2i+1 < dims,
+ * turned by pos[t] * freq[i]]. */
+int mi355_latent_kv_append(int64_t tokens, int rank, int rot, const void* src, int src_dt, int64_t ld, const float* w, float eps, const int* pos,
+                           const int* dst_row, const float* freq, int dims, void* cache, int cache_dt, int64_t ldc, void* stream);
+/* dst[t, h * dst_hs + dst_off + i] = src[t, h * src_hs + src_off + i] for i < n (dst fp32), the pairs of [rot_start, rot_start + dims) turned by
+ * pos[t] * freq[i] (interleaved rotary embedding). */
+int mi355_rope_heads(int64_t tokens, int H, int n, const void* src, int src_dt, int64_t ld_src, int src_hs, int src_off, float* dst, int64_t ld_dst,
+                     int dst_hs, int dst_off, int rot_start, int dims, const float* freq, const int* pos, void* stream);
+/* out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * w * silu(gate[t, h, :]); o fp32 [tokens, H * D], w fp32 [D]. */
+int mi355_gated_headnorm(int64_t tokens, int H, int D, const float* o, const float* w, const void* gate, int g_dt, int64_t ldg, float eps, void* out,
+                         int out_dt, int64_t ldo, void* stream);
+/* Gated linear attention over the rows [seq_off[s], seq_off[s+1]) of each sequence s, state[slot[s]] (fp32 [H, dk, dv]) read and written:
+ * S <- diag(a_t) S + k_t v_t^T, o_t = S^T (q_t * qscale), a_t = sigmoid(z_t + zbias)^inv_tau.  q / k rows [H * dk], v rows [H * dv] of dtype dt, z rows [H * dk] of dtype z_dt,
+ * o fp32 [tokens, H * dv].  dk <= 256. */
+int mi355_gla_fwd(int n_seq, const int* seq_off, const int* slot, int H, int dk, int dv, const void* q, const void* k, const void* v, const void* z, int dt,
+                  int z_dt, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldz, const float* zbias, float inv_tau, float qscale, float* state, float* o, void* stream);
+/* Grouped sigmoid router: s = sigmoid(logits), choice = s + correction (may be NULL); a group (E / groups neighbours) scores the sum of its two
+ * largest choices, experts outside the `keep` best groups are excluded, the `top` largest choices win; wts = s / (sum + 1e-20) * scale.
+ * ids int32 [tokens, top] in descending order of choice, wts fp32 [tokens, top]. */
+int mi355_moe_route(int64_t tokens, int E, int top, int groups, int keep, const float* logits, const float* correction, float scale, int* ids, float* wts,
+                    void* stream);
+/* Dispatch lists of `entries` = tokens * top choices: offs int32 [E + 1], perm int32 [entries] = the entries sorted by expert (token order inside one). */
+int mi355_moe_dispatch(int64_t entries, int E, const int* ids, int* offs, int* perm, void* stream);
+/* C[b][m, n] = epi(sum_k A[b][m, k] B[b][n, k]) with general strides: A at b * a_bs + row * lda + k, B at b * b_bs + n * sbn + k * sbk (one of sbn / sbk
+ * is 1), C at b * c_bs + row * ldc + n.  grp_offs (may be NULL): batch b owns the sorted rows [grp_offs[b], grp_offs[b+1]) and M bounds their number;
+ * a_rows: sorted row r reads A row a_rows[r] / a_div; c_rows: it writes C row c_rows[r]; row_scale: that C row is scaled.  epi 1 = relu(x)^2.
+ * use_mfma needs bf16 A and B; otherwise fp32 FMA accumulation in a fixed k order. */
+int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t lda, int64_t a_bs, const void* B, int b_dt, int64_t sbn, int64_t sbk,
+                int64_t b_bs, void* C, int c_dt, int64_t ldc, int64_t c_bs, const int* grp_offs, const int* a_rows, int a_div, const int* c_rows,
+                const float* row_scale, int epi, int use_mfma, void* stream);
+/* Causal attention with two-part keys over ragged batches: sequence s has n_new[s] query rows starting at row q_row0[s], `past[s]` earlier keys;
+ * key j of it is K1 row k1_row0[s] + j (head stride k1_hs, D1 wide), K2 row k2_row0[s] + j (shared by heads, D2 wide), value row v_row0[s] + j.
+ * Q fp32 [.., H, D1 + D2]; K1 / K2 / V / O of dtype dt.  A tile covers 32 / hm tokens x hm heads (hm > 1 needs k1_hs == v_hs == 0). */
+int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, int D2, int DV, const float* Q, int64_t ldq, int q_hs, const void* K1, int64_t ldk1,
+                      int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
+                      const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
+                      int use_mfma, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

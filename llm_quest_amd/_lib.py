@@ -12,6 +12,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("MI355_LIB_PATH") or os.path.join(_HERE, "libmi355vlm.so")  # override: profiling builds only
+SERVE_LIB_PATH = os.path.join(_HERE, "libmi355serve.so")  # `make serve`: the objects of the serving path only; used when the full library is not built
 CSRC = os.path.join(_HERE, "csrc")
 
 DT_BF16, DT_F32, DT_SPLIT3 = 0, 1, 2  # DT_SPLIT3: an fp32 value as bf16 [hi | lo | hi] column blocks (include/mi355_vlm.h)
@@ -98,6 +99,18 @@ SIGNATURES = {
     "mi355_attn_decode": [_I, _I, _I, _I, _P, _P, _P, _L, _L, _I, _P, _P, _L, _P, _F, _I, _P, _P],
     "mi355_kv_append": [_I, _I, _P, _L, _P, _L, _P, _P, _L, _L, _I, _P, _P],
     "mi355_argmax_rows": [_L, _L, _P, _L, _P, _P, _P],
+    # ragged-batch serving of hybrid decoders (csrc/seqmix.hip, csrc/bgemm.hip, csrc/latent_attn.hip)
+    "mi355_embed_hash_fwd": [_L, _I, _I, _P, _P, _P, _F, _P, _I, _I, _I, _P, _P],
+    "mi355_add_layernorm_fwd": [_L, _I, _P, _F, _P, _I, _L, _I, _P, _P, _F, _P, _P, _I, _P],
+    "mi355_rmsnorm_rows": [_L, _I, _P, _I, _L, _P, _F, _P, _I, _L, _P],
+    "mi355_latent_kv_append": [_L, _I, _I, _P, _I, _L, _P, _F, _P, _P, _P, _I, _P, _I, _L, _P],
+    "mi355_rope_heads": [_L, _I, _I, _P, _I, _L, _I, _I, _P, _L, _I, _I, _I, _I, _P, _P, _P],
+    "mi355_gated_headnorm": [_L, _I, _I, _P, _P, _P, _I, _L, _F, _P, _I, _L, _P],
+    "mi355_gla_fwd": [_I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _I, _L, _L, _L, _L, _P, _F, _F, _P, _P, _P],
+    "mi355_moe_route": [_L, _I, _I, _I, _I, _P, _P, _F, _P, _P, _P],
+    "mi355_moe_dispatch": [_L, _I, _P, _P, _P, _P],
+    "mi355_bgemm": [_I, _I, _I, _I, _P, _I, _L, _L, _P, _I, _L, _L, _L, _P, _I, _L, _L, _P, _P, _I, _P, _P, _I, _I, _P],
+    "mi355_latent_attn": [_I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _F, _I, _P],
     # measurement aid (csrc/probe.hip)
     "mi355_mfma_pipe_probe": [_I, _I, _P, _P],
     # stand-alone RoPE and dropout (csrc/rope_dropout.hip, csrc/attention_generic.hip)
@@ -137,21 +150,34 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
+    path, partial = LIB_PATH, False
+    if not os.path.exists(path) and os.path.exists(SERVE_LIB_PATH):
+        path, partial = SERVE_LIB_PATH, True  # entry points outside the serving path are absent: calling one raises AttributeError
+    if not os.path.exists(path):
         raise RuntimeError(
             f"{LIB_PATH} is missing: the HIP extension is the only implementation of this path "
             "(no CPU fallback). Build it with `python -c 'import __graft_entry__ as g; g.build()'`."
         )
-    lib = ctypes.CDLL(LIB_PATH)
+    lib = ctypes.CDLL(path)
     lib.mi355_last_error.restype = ctypes.c_char_p
     lib.mi355_last_error.argtypes = []
     lib.mi355_abi_version.restype = ctypes.c_int
     for name, argtypes in SIGNATURES.items():
-        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        try:
+            fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        except AttributeError:
+            if partial:
+                continue
+            raise
         fn.argtypes = argtypes
         fn.restype = ctypes.c_int
     for name, (argtypes, restype) in QUERIES.items():
-        fn = getattr(lib, name)
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            if partial:
+                continue
+            raise
         fn.argtypes = argtypes
         fn.restype = restype
     _lib = lib

@@ -1,0 +1,213 @@
+"""Token mixers and the routed feed-forward of hybrid decoders served in ragged batches, as modules whose constants are constructor arguments:
+
+* ``LatentAttention``       -- multi-head latent attention: queries and keys / values go through low-rank latents, one rotated key part is shared by all
+  heads, only the normalised latent and that rotated part are cached (optionally another layer's);
+* ``GatedLinearAttention``  -- linear attention with a per-key-channel decay and a matrix state per head, carried in fp32;
+* ``GroupedSigmoidMoE``     -- sigmoid-scored experts chosen inside the best groups, squared-ReLU experts.
+
+They run one *step* of a batch (``SeqStep``): the new tokens of every sequence, packed row after row, against what ``utils.SlotStateCache`` holds.  Inference
+only, HIP kernels only (``kernels_seq``); weights are bf16, what is normalised, rotated, decayed, accumulated over time or routed is fp32.
+"""
+
+import torch
+import torch.nn as nn
+
+from llm_quest_amd import _lib as L
+from llm_quest_amd import kernels_seq as S
+
+BF16, F32, I32 = torch.bfloat16, torch.float32, torch.int32
+
+
+class SeqStep:
+    """One step of a ragged batch: ``entries`` = [(slot, new tokens)], the cache gives every sequence's length and last token.  Holds the device-side
+    descriptors the kernels read.  ``fresh``: every sequence starts at its first token (prompts; attention may rebuild keys and values from this step's rows)."""
+
+    def __init__(self, cache, entries, device, act_dtype):
+        self.cache, self.act_dtype, self.device = cache, act_dtype, device
+        tok, prev, pos, seq_off, slots, past, n_new = [], [], [], [0], [], [], []
+        for slot, new in entries:
+            if len(new) == 0:
+                raise ValueError("SeqStep: a sequence of the step brings no token")
+            start = cache.length[slot]
+            tok.extend(new)
+            prev.append(cache.last_token[slot])
+            prev.extend(new[:-1])
+            pos.extend(range(start, start + len(new)))
+            seq_off.append(seq_off[-1] + len(new))
+            slots.append(slot)
+            past.append(start)
+            n_new.append(len(new))
+        cache.reserve(max(p + n for p, n in zip(past, n_new)))
+        cap = cache.capacity
+        self.T, self.n_seq, self.max_new = len(tok), len(slots), max(n_new)
+        self.fresh = all(p == 0 for p in past)
+        self.host_seq_off = seq_off
+        row0 = [s * cap for s in slots]
+        dst = [row0[i] + p for i in range(len(slots)) for p in range(past[i], past[i] + n_new[i])]
+        # one host-to-device copy for all descriptors
+        flat = tok + prev + pos + dst + seq_off + slots + past + n_new + row0 + list(range(self.T))
+        buf = torch.tensor(flat, dtype=I32).to(device, non_blocking=False)
+        T, n = self.T, self.n_seq
+        cuts = [T, T, T, T, n + 1, n, n, n, n, T]
+        parts, at = [], 0
+        for c in cuts:
+            parts.append(buf[at : at + c])
+            at += c
+        (self.tok, self.prev, self.pos, self.dst_row, self.seq_off, self.slots, self.past, self.n_new, self.cache_row0, self.local_row) = parts
+        self.q_row0 = self.seq_off[:n]
+        self.local = {}  # layer -> this step's latent rows [T, rank + rot] (prompts: the expanded form reads them instead of the cache)
+
+
+def _f32(t):
+    return None if t is None else t.detach().to(F32).contiguous()
+
+
+class _Frozen(nn.Module):
+    """Inference-only module: bf16 parameters without gradients; fp32 copies of the small vectors are made once per device (``prepare``)."""
+
+    def _param(self, *shape):
+        return nn.Parameter(torch.zeros(*shape, dtype=BF16), requires_grad=False)
+
+
+class LatentAttention(_Frozen):
+    """Multi-head latent attention.  Per head ``dim`` unrotated + ``rot_dim`` rotated query / key entries, ``vdim`` values; latents of ``q_rank`` /
+    ``kv_rank``.  ``kv_from``: read that layer's cached rows instead of projecting own ones.  Rotary: interleaved pairs, ``rot_dims`` of the rotated part
+    turn (base ``rot_base``)."""
+
+    def __init__(self, width, heads, dim, rot_dim, vdim, q_rank, kv_rank, scale, rot_dims, rot_base, eps, layer_idx, kv_from=None):
+        super().__init__()
+        self.width, self.heads, self.dim, self.rot_dim, self.vdim = width, heads, dim, rot_dim, vdim
+        self.q_rank, self.kv_rank, self.scale, self.rot_dims, self.rot_base, self.eps = q_rank, kv_rank, float(scale), rot_dims, float(rot_base), float(eps)
+        self.layer_idx, self.kv_from = layer_idx, kv_from
+        own = kv_from is None
+        # down projections side by side: [q_rank | kv_rank + rot_dim] rows -> one product
+        self.w_down = self._param(q_rank + (kv_rank + rot_dim if own else 0), width)
+        self.q_norm = self._param(q_rank)
+        self.kv_norm = self._param(kv_rank) if own else None
+        self.w_uq = self._param(heads * (dim + rot_dim), q_rank)
+        self.w_ukv = self._param(heads * (dim + vdim), kv_rank)  # [key up-projection | value up-projection] rows
+        self.w_o = self._param(width, heads * vdim)
+        self._ready = None
+
+    def cache_spec(self):
+        return ("rows", self.kv_rank + self.rot_dim) if self.kv_from is None else ("shared", self.kv_from)
+
+    def prepare(self, device):
+        if self._ready != device:
+            self.q_norm32 = _f32(self.q_norm)
+            self.kv_norm32 = _f32(self.kv_norm)
+            self.freq = S.rope_frequencies(self.rot_dims, self.rot_base, device)
+            self._ready = device
+
+    @torch.no_grad()
+    def step(self, h, st):
+        """h [T, width] in the activation dtype -> the mixer's output rows [T, width]."""
+        self.prepare(h.device)
+        H, dn, dr, dv, R, Rq = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank, self.q_rank
+        own = self.kv_from is None
+        src = self.layer_idx if own else self.kv_from
+        cache2d = st.cache.rows2d(self.layer_idx)
+        down = S.linear(h, self.w_down)
+        q = S.linear(S.rmsnorm_rows(down[:, :Rq], self.q_norm32, self.eps), self.w_uq)
+        if own:
+            S.latent_kv_append(down[:, Rq:], R, dr, self.kv_norm32, self.eps, st.pos, st.dst_row, self.freq, self.rot_dims, cache2d)
+        T = h.shape[0]
+        if st.fresh:
+            # prompts: keys and values per head rebuilt from this step's latent rows, ordinary head-by-head attention
+            if own:
+                lat = torch.empty((T, R + dr), dtype=st.act_dtype, device=h.device)
+                S.latent_kv_append(down[:, Rq:], R, dr, self.kv_norm32, self.eps, st.pos, st.local_row, self.freq, self.rot_dims, lat)
+                st.local[src] = lat
+            lat = st.local[src]
+            kv = S.linear(lat[:, :R], self.w_ukv)  # [T, H*dn | H*dv]
+            q32 = torch.empty((T, H * (dn + dr)), dtype=F32, device=h.device)
+            S.rope_heads(q, H, dn + dr, dn + dr, 0, q32, dn + dr, 0, dn, self.rot_dims, self.freq, st.pos)
+            ctx = torch.empty((T, H * dv), dtype=st.act_dtype, device=h.device)
+            S.latent_attn(q32, kv[:, : H * dn], lat[:, R:], kv[:, H * dn :], ctx, H, 1, dn, dr, dv, dn + dr, dn, dv, dv,
+                          (st.q_row0, st.n_new, st.past, st.q_row0, st.q_row0, st.q_row0), st.max_new, self.scale)
+        else:
+            # continuation: the key up-projection folded onto the query, the value up-projection applied after the attention -- the cache rows are
+            # keys and values of every head as they stand
+            qf = torch.empty((T, H * (R + dr)), dtype=F32, device=h.device)
+            S.bgemm(q, self.w_ukv, qf, T, R, dn, batch=H, lda=q.stride(0), a_bs=dn + dr, sbn=1, sbk=R, b_bs=dn * R, ldc=H * (R + dr), c_bs=R + dr)
+            S.rope_heads(q, H, dr, dn + dr, dn, qf, R + dr, R, 0, self.rot_dims, self.freq, st.pos)
+            hm = 1
+            while hm < min(H, 32):
+                hm *= 2
+            ol = torch.empty((T, H * R), dtype=st.act_dtype, device=h.device)
+            S.latent_attn(qf, cache2d, cache2d[:, R:], cache2d, ol, H, hm, R, dr, R, R + dr, 0, 0, R,
+                          (st.q_row0, st.n_new, st.past, st.cache_row0, st.cache_row0, st.cache_row0), st.max_new, self.scale)
+            ctx = torch.empty((T, H * dv), dtype=st.act_dtype, device=h.device)
+            S.bgemm(ol, self.w_ukv[H * dn :], ctx, T, dv, R, batch=H, lda=H * R, a_bs=R, sbn=R, sbk=1, b_bs=dv * R, ldc=H * dv, c_bs=dv)
+        return S.linear(ctx, self.w_o)
+
+
+class GatedLinearAttention(_Frozen):
+    """Per head a state S [dim, vdim]: S <- diag(a) S + k v^T, o = S^T q with q scaled by dim^-1/2; a = sigmoid(z)^(1/tau) per key channel, z from a
+    low-rank projection with bias.  o is RMS-normed per head (one weight [vdim] for all heads), gated by silu of a projection, and projected out."""
+
+    def __init__(self, width, heads, dim, vdim, decay_rank, tau, eps, layer_idx):
+        super().__init__()
+        self.width, self.heads, self.dim, self.vdim, self.decay_rank, self.tau, self.eps, self.layer_idx = width, heads, dim, vdim, decay_rank, float(tau), float(eps), layer_idx
+        # [q | k | v | gate | decay down-projection] rows -> one product
+        self.w_in = self._param(2 * heads * dim + 2 * heads * vdim + decay_rank, width)
+        self.w_a2 = self._param(heads * dim, decay_rank)
+        self.a2_bias = self._param(heads * dim)
+        self.norm = self._param(vdim)
+        self.w_o = self._param(width, heads * vdim)
+        self._ready = None
+
+    def cache_spec(self):
+        return ("state", (self.heads, self.dim, self.vdim))
+
+    def prepare(self, device):
+        if self._ready != device:
+            self.a2_bias32, self.norm32 = _f32(self.a2_bias), _f32(self.norm)
+            self._ready = device
+
+    @torch.no_grad()
+    def step(self, h, st):
+        self.prepare(h.device)
+        H, dk, dv = self.heads, self.dim, self.vdim
+        proj = S.linear(h, self.w_in)
+        a, b, c = H * dk, 2 * H * dk, 2 * H * dk + H * dv
+        z = S.linear(proj[:, c + H * dv :], self.w_a2, out_dtype=F32)
+        o = S.gla(proj[:, :a], proj[:, a:b], proj[:, b:c], z, self.a2_bias32, 1.0 / self.tau, dk ** -0.5, st.seq_off, st.slots, st.cache.state(self.layer_idx), H, dk, dv)
+        mix = S.gated_headnorm(o, self.norm32, proj[:, c : c + H * dv], H, dv, self.eps, st.act_dtype)
+        return S.linear(mix, self.w_o)
+
+
+class GroupedSigmoidMoE(_Frozen):
+    """``experts`` feed-forward experts (down(relu(up x)^2), no biases), ``top`` per token.  Scores sigmoid(router x); the choice adds a per-expert
+    correction; experts form ``groups`` runs of neighbours of which the ``keep`` best (by the sum of their two largest choice scores) stay eligible;
+    weights are the winners' uncorrected scores, normalised and multiplied by ``scale``.  Returns the experts' weighted outputs as ``top`` fp32 rows per
+    token, in descending order of the choice score: the sum is taken by the norm kernel that follows."""
+
+    def __init__(self, width, ff, experts, top, groups, keep, scale, correction=True):
+        super().__init__()
+        self.width, self.ff, self.experts, self.top, self.groups, self.keep, self.scale = width, ff, experts, top, groups, keep, float(scale)
+        self.w_router = self._param(experts, width)
+        self.correction = nn.Parameter(torch.zeros(experts, dtype=BF16), requires_grad=False) if correction else None
+        self.w_up = self._param(experts, ff, width)
+        self.w_down = self._param(experts, width, ff)
+        self._ready = None
+
+    def prepare(self, device):
+        if self._ready != device:
+            self.correction32 = _f32(self.correction)
+            self._ready = device
+
+    @torch.no_grad()
+    def step(self, x32, h):
+        """x32: the fp32 residual rows (the router reads them), h: the same rows in the activation dtype -> fp32 [T * top, width]."""
+        self.prepare(h.device)
+        T, E, top = h.shape[0], self.experts, self.top
+        logits = torch.empty((T, E), dtype=F32, device=h.device)
+        S.bgemm(x32, self.w_router, logits, T, E, self.width, mfma=False)
+        ids, wts = S.moe_route(logits, self.correction32, top, self.groups, self.keep, self.scale)
+        offs, perm = S.moe_dispatch(ids.view(-1), E)
+        act = torch.empty((T * top, self.ff), dtype=h.dtype, device=h.device)
+        S.bgemm(h, self.w_up, act, T * top, self.ff, self.width, batch=E, sbn=self.width, b_bs=self.ff * self.width, grp_offs=offs, a_rows=perm, a_div=top, epi=1)
+        out = torch.empty((T * top, self.width), dtype=F32, device=h.device)
+        S.bgemm(act, self.w_down, out, T * top, self.width, self.ff, batch=E, sbn=self.ff, b_bs=self.width * self.ff, grp_offs=offs, c_rows=perm, row_scale=wts.view(-1))
+        return out

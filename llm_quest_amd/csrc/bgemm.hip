@@ -1,0 +1,230 @@
+// Batched / grouped matrix products with general strides (gfx950 only).
+//
+//   C[b][m, n] = epi( sum_k A[b][m, k] * B[b][n, k] )        b < batch
+//
+// A element (m, k) of batch b:  A[b * a_bs + row(m) * lda + k]
+// B element (n, k) of batch b:  B[b * b_bs + n * sbn + k * sbk]      (sbk == 1: weight stored [out, in]; sbn == 1: stored [in, out])
+// C element (m, n) of batch b:  C[b * c_bs + crow(m) * ldc + n]
+//
+// Uses: the per-head products of latent attention with the key / value up-projections folded onto the query and the output side;
+// the experts of a mixture (batch = expert, a batch's rows given by device-side offsets, A rows gathered through a dispatch list,
+// C rows scattered back and scaled by the routing weight); and every linear layer of the true-fp32 mode (fp32 activations,
+// weights kept in bf16 -- exactly representable -- and widened on load, fp32 FMA accumulation in a fixed k order, so a row's result does not depend
+// on which other rows share its tile).
+//
+// Two compute paths:
+//   * FMA: 64 x 64 tile, 256 threads, 4 x 4 outputs per thread, k in steps of 16 through LDS (any operand type);
+//   * MFMA (bf16 A and B): the same tile, four waves of 32 x 32 on v_mfma_f32_32x32x8_bf16_1k, k in steps of 32.
+#include "common.h"
+
+#define ST(s) ((hipStream_t)(s))
+
+struct BgemmArgs {
+    const void* A;
+    const void* B;
+    void* C;
+    int64_t lda, a_bs, sbn, sbk, b_bs, ldc, c_bs;
+    int M, N, K;
+    const int* grp_offs;     // [batch + 1] or null: rows of batch b are the sorted rows [grp_offs[b], grp_offs[b+1]) (then M is the tile bound)
+    const int* a_rows;       // or null: sorted row r reads A row a_rows[r] / a_div
+    int a_div;
+    const int* c_rows;       // or null: sorted row r writes C row c_rows[r]
+    const float* row_scale;  // or null: C row (after c_rows) is multiplied by row_scale[that row]
+    int epi;                 // 0 none, 1 relu(x)^2
+    int a_dt, b_dt, c_dt;
+};
+
+__device__ __forceinline__ float ldx(const void* p, int dt, int64_t i) { return dt == MI355_DT_F32 ? ((const float*)p)[i] : bf2f(((const bf16_t*)p)[i]); }
+
+#define BM 64
+#define BN 64
+#define BK 16
+
+__global__ __launch_bounds__(256) void bgemm_fma_kernel(BgemmArgs p) {
+    __shared__ float As[BK][BM + 4];
+    __shared__ float Bs[BK][BN + 4];
+    const int b = blockIdx.z;
+    int row0 = 0, rows = p.M;
+    if (p.grp_offs) {
+        row0 = p.grp_offs[b];
+        rows = p.grp_offs[b + 1] - row0;
+    }
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    if (m0 >= rows) return;
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    // loader roles: A element (m = tid / 4 + {0}, k = (tid % 4) * 4 .. +4): 64 rows x 16 k
+    const int am = tid >> 2, ak = (tid & 3) * 4;
+    int64_t a_base = -1;
+    if (m0 + am < rows) {
+        const int r = row0 + m0 + am;
+        const int64_t arow = p.a_rows ? p.a_rows[r] / p.a_div : r;
+        a_base = (int64_t)b * p.a_bs + arow * p.lda;
+    }
+    // B loader: if sbk == 1 the same (n = tid / 4, k chunk) shape as A; if sbn == 1, n runs fastest: (k = tid / 16, n = (tid % 16) * 4 .. +4)
+    const bool b_kfast = p.sbk == 1;
+    const int bn = b_kfast ? tid >> 2 : (tid & 15) * 4, bk = b_kfast ? (tid & 3) * 4 : tid >> 4;
+    const int64_t b_base = (int64_t)b * p.b_bs;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < p.K; k0 += BK) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int k = k0 + ak + i;
+            As[ak + i][am] = (a_base >= 0 && k < p.K) ? ldx(p.A, p.a_dt, a_base + k) : 0.f;
+        }
+        if (b_kfast) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int k = k0 + bk + i, n = n0 + bn;
+                Bs[bk + i][bn] = (n < p.N && k < p.K) ? ldx(p.B, p.b_dt, b_base + (int64_t)n * p.sbn + k) : 0.f;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int k = k0 + bk, n = n0 + bn + i;
+                Bs[bk][bn + i] = (n < p.N && k < p.K) ? ldx(p.B, p.b_dt, b_base + (int64_t)n * p.sbn + (int64_t)k * p.sbk) : 0.f;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BK; ++k) {
+            float a[4], bb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i], bb[i] = Bs[k][tx * 4 + i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], bb[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= rows) continue;
+        const int r = row0 + m;
+        const int64_t crow = p.c_rows ? p.c_rows[r] : r;
+        const float sc = p.row_scale ? p.row_scale[crow] : 1.0f;
+        const int64_t cb = (int64_t)b * p.c_bs + crow * p.ldc;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= p.N) continue;
+            float v = acc[i][j];
+            if (p.epi == 1) v = v > 0.f ? v * v : 0.f;
+            v *= sc;
+            if (p.c_dt == MI355_DT_F32) ((float*)p.C)[cb + n] = v;
+            else ((bf16_t*)p.C)[cb + n] = f2bf(v);
+        }
+    }
+}
+
+// ---- MFMA path: bf16 A and B.  LDS tiles [64][32 + 8] bf16 (k contiguous; the 16-byte pad keeps the 8-byte fragment reads off one bank group).
+// Wave w computes the 32 x 32 block (w / 2, w % 2).  v_mfma_f32_32x32x8_bf16_1k: lane l supplies A[m = l % 32][k = 4 * (l / 32) .. +4] and
+// B[n = l % 32][same k]; accumulator register 4 * g + i of lane l is C[m = 8 * g + 4 * (l / 32) + i][n = l % 32].
+#define MK 32
+#define MPAD 8
+__global__ __launch_bounds__(256) void bgemm_mfma_kernel(BgemmArgs p) {
+    __shared__ bf16_t As[BM][MK + MPAD];
+    __shared__ bf16_t Bs[BN][MK + MPAD];
+    const int b = blockIdx.z;
+    int row0 = 0, rows = p.M;
+    if (p.grp_offs) {
+        row0 = p.grp_offs[b];
+        rows = p.grp_offs[b + 1] - row0;
+    }
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    if (m0 >= rows) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bf16_t* A = (const bf16_t*)p.A;
+    const bf16_t* B = (const bf16_t*)p.B;
+    // loaders: 64 rows x 32 k = 2048 elements, 8 per thread: (row = tid / 4, k = (tid % 4) * 8 .. +8)
+    const int lr = tid >> 2, lk = (tid & 3) * 8;
+    int64_t a_base = -1;
+    if (m0 + lr < rows) {
+        const int r = row0 + m0 + lr;
+        const int64_t arow = p.a_rows ? p.a_rows[r] / p.a_div : r;
+        a_base = (int64_t)b * p.a_bs + arow * p.lda;
+    }
+    const bool b_kfast = p.sbk == 1;
+    const int64_t b_base = (int64_t)b * p.b_bs;
+    const bool a_vec = (p.lda % 8 == 0) && (p.a_bs % 8 == 0) && (((uintptr_t)p.A & 15) == 0);
+    const bool b_vec = b_kfast && (p.sbn % 8 == 0) && (p.b_bs % 8 == 0) && (((uintptr_t)p.B & 15) == 0);
+    f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+    for (int k0 = 0; k0 < p.K; k0 += MK) {
+        // A tile
+        if (a_base >= 0 && a_vec && k0 + lk + 8 <= p.K) {
+            *(u32x4*)&As[lr][lk] = *(const u32x4*)(A + a_base + k0 + lk);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) As[lr][lk + i] = (a_base >= 0 && k0 + lk + i < p.K) ? A[a_base + k0 + lk + i] : (bf16_t)0;
+        }
+        // B tile
+        if (b_kfast) {
+            const int n = n0 + lr;
+            if (n < p.N && b_vec && k0 + lk + 8 <= p.K) {
+                *(u32x4*)&Bs[lr][lk] = *(const u32x4*)(B + b_base + (int64_t)n * p.sbn + k0 + lk);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) Bs[lr][lk + i] = (n < p.N && k0 + lk + i < p.K) ? B[b_base + (int64_t)n * p.sbn + k0 + lk + i] : (bf16_t)0;
+            }
+        } else {  // n runs fastest in memory: thread (k = tid / 8, n = (tid % 8) * 8 .. +8)
+            const int k = k0 + (tid >> 3), nb = (tid & 7) * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int n = n0 + nb + i;
+                Bs[nb + i][tid >> 3] = (n < p.N && k < p.K) ? B[b_base + (int64_t)n * p.sbn + (int64_t)k * p.sbk] : (bf16_t)0;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < MK; kk += 8) {
+            const bf16x4 a = *(const bf16x4*)&As[wm + (lane & 31)][kk + 4 * (lane >> 5)];
+            const bf16x4 bb = *(const bf16x4*)&Bs[wn + (lane & 31)][kk + 4 * (lane >> 5)];
+            acc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a, bb, acc, 0, 0, 0);
+        }
+        __syncthreads();
+    }
+    const int n = n0 + wn + (lane & 31);
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = m0 + wm + 8 * g + 4 * (lane >> 5) + i;
+            if (m >= rows || n >= p.N) continue;
+            const int r = row0 + m;
+            const int64_t crow = p.c_rows ? p.c_rows[r] : r;
+            const float sc = p.row_scale ? p.row_scale[crow] : 1.0f;
+            float v = acc[4 * g + i];
+            if (p.epi == 1) v = v > 0.f ? v * v : 0.f;
+            v *= sc;
+            const int64_t ci = (int64_t)b * p.c_bs + crow * p.ldc + n;
+            if (p.c_dt == MI355_DT_F32) ((float*)p.C)[ci] = v;
+            else ((bf16_t*)p.C)[ci] = f2bf(v);
+        }
+}
+
+extern "C" int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t lda, int64_t a_bs, const void* B, int b_dt, int64_t sbn, int64_t sbk,
+                           int64_t b_bs, void* C, int c_dt, int64_t ldc, int64_t c_bs, const int* grp_offs, const int* a_rows, int a_div, const int* c_rows,
+                           const float* row_scale, int epi, int use_mfma, void* stream) {
+    MI355_REQUIRE(batch > 0 && batch <= 65535 && M > 0 && N > 0 && K > 0 && A && B && C, "bgemm: bad arguments");
+    MI355_REQUIRE((a_dt == MI355_DT_BF16 || a_dt == MI355_DT_F32) && (b_dt == MI355_DT_BF16 || b_dt == MI355_DT_F32) && (c_dt == MI355_DT_BF16 || c_dt == MI355_DT_F32),
+                  "bgemm: bad dtype");
+    MI355_REQUIRE(epi == 0 || epi == 1, "bgemm: bad epilogue");
+    MI355_REQUIRE(!a_rows || a_div >= 1, "bgemm: gathered rows need a divisor >= 1");
+    MI355_REQUIRE(sbn >= 1 && sbk >= 1 && (sbn == 1 || sbk == 1), "bgemm: one of B's strides must be 1");
+    MI355_REQUIRE(!use_mfma || (a_dt == MI355_DT_BF16 && b_dt == MI355_DT_BF16), "bgemm: the MFMA path takes bf16 operands");
+    BgemmArgs p;
+    p.A = A, p.B = B, p.C = C;
+    p.lda = lda, p.a_bs = a_bs, p.sbn = sbn, p.sbk = sbk, p.b_bs = b_bs, p.ldc = ldc, p.c_bs = c_bs;
+    p.M = M, p.N = N, p.K = K;
+    p.grp_offs = grp_offs, p.a_rows = a_rows, p.a_div = a_rows ? a_div : 1, p.c_rows = c_rows, p.row_scale = row_scale;
+    p.epi = epi, p.a_dt = a_dt, p.b_dt = b_dt, p.c_dt = c_dt;
+    const int64_t my = ((int64_t)M + BM - 1) / BM;
+    MI355_REQUIRE(my <= 65535, "bgemm: too many row tiles");
+    const dim3 grid((N + BN - 1) / BN, (unsigned)my, batch);
+    if (use_mfma) bgemm_mfma_kernel<<<grid, 256, 0, ST(stream)>>>(p);
+    else bgemm_fma_kernel<<<grid, 256, 0, ST(stream)>>>(p);
+    MI355_LAUNCH_CHECK("bgemm");
+    return 0;
+}

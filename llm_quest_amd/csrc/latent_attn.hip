@@ -1,0 +1,197 @@
+// Causal softmax attention whose keys come in two parts -- a main part (per head, or one shared by all heads) and a rotated part shared by
+// all heads -- over ragged batches (gfx950 only).  It serves multi-head latent attention in both of its forms:
+//   * expanded (prompts): K1 = the per-head keys and V = the per-head values rebuilt from the latent rows of this step, K2 = the rotated key part;
+//   * folded (one-token steps): the key up-projection is folded into the query and the value up-projection is applied after the attention, so
+//     K1 = V = the cached latent rows themselves (head stride 0), K2 = the cached rotated part: the cache is read once for all heads.
+//
+// score(row, j) = scale * ( Q[row, :D1] . K1[j, head, :] + Q[row, D1:] . K2[j, :] ),  softmax over j <= past + token index, out = sum_j p V[j].
+// Scores, softmax statistics and the output accumulators are fp32.  A tile is `tm` tokens x `hm` heads = 32 query rows (hm > 1 only with shared
+// keys and values) against 64 keys at a time.
+//
+// Two compute paths: fp32 FMA through LDS (any operand type: the true-fp32 mode), and bf16 MFMA (v_mfma_f32_32x32x8_bf16_1k) for bf16 keys / values.
+#include "common.h"
+
+#define ST(s) ((hipStream_t)(s))
+
+struct LatAttnArgs {
+    const float* Q;
+    const void* K1;
+    const void* K2;
+    const void* V;
+    void* O;
+    int64_t ldq, ldk1, ldk2, ldv, ldo;
+    int q_hs, k1_hs, v_hs, o_hs;
+    int D1, D2, DV, H, hm, dt;
+    const int *q_row0, *n_new, *past, *k1_row0, *k2_row0, *v_row0;
+    float scale;
+};
+
+__device__ __forceinline__ float lda_dt(const void* p, int dt, int64_t i) { return dt == MI355_DT_F32 ? ((const float*)p)[i] : bf2f(((const bf16_t*)p)[i]); }
+
+#define AM 32  // query rows per tile
+#define AN 64  // keys per step
+#define AC 32  // feature chunk of the score product
+
+template <int NC>
+__global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
+    __shared__ float Qs[AM][AC + 1];
+    __shared__ float Ks[AN][AC + 1];
+    __shared__ float Ps[AM][AN + 4];
+    __shared__ float fs[AM], ls[AM];
+    const int s = blockIdx.z, tm = AM / p.hm;
+    const int tok0 = blockIdx.x * tm, head0 = blockIdx.y * p.hm;
+    const int n_new = p.n_new[s], past = p.past[s];
+    if (tok0 >= n_new) return;
+    const int64_t qr0 = p.q_row0[s], k1r0 = p.k1_row0[s], k2r0 = p.k2_row0[s], vr0 = p.v_row0[s];
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int DK = p.D1 + p.D2;
+    const int n_keys = past + min(tok0 + tm, n_new);  // keys any row of the tile may see
+    // S layout: rows 2 ty, 2 ty + 1; keys tx + 16 i
+    int lim[2];
+    float m_run[2] = {-__builtin_huge_valf(), -__builtin_huge_valf()}, l_run[2] = {0.f, 0.f};
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+        const int r = 2 * ty + a, tok = tok0 + r / p.hm, head = head0 + r % p.hm;
+        lim[a] = (tok < n_new && head < p.H) ? past + tok : -1;
+    }
+    // PV layout: rows 8 rg .. +8, columns c + 64 i
+    const int rg = tid >> 6, c = tid & 63;
+    float o[8][NC];
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+#pragma unroll
+        for (int i = 0; i < NC; ++i) o[r][i] = 0.f;
+
+    for (int j0 = 0; j0 < n_keys; j0 += AN) {
+        float acc[2][4] = {};
+        for (int d0 = 0; d0 < DK; d0 += AC) {
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {  // Q chunk: 32 rows x 32 features
+                const int e = tid + 256 * i, d = d0 + (e & 31), r = e >> 5;
+                const int tok = tok0 + r / p.hm, head = head0 + r % p.hm;
+                Qs[r][e & 31] = (d < DK && tok < n_new && head < p.H) ? p.Q[(qr0 + tok) * p.ldq + (int64_t)head * p.q_hs + d] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {  // K chunk: 64 keys x 32 features
+                const int e = tid + 256 * i, d = d0 + (e & 31), j = j0 + (e >> 5);
+                float v = 0.f;
+                if (j < n_keys && d < DK)
+                    v = d < p.D1 ? lda_dt(p.K1, p.dt, (k1r0 + j) * p.ldk1 + (int64_t)head0 * p.k1_hs + d) : lda_dt(p.K2, p.dt, (k2r0 + j) * p.ldk2 + (d - p.D1));
+                Ks[e >> 5][e & 31] = v;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int d = 0; d < AC; ++d) {
+                const float q0 = Qs[2 * ty][d], q1 = Qs[2 * ty + 1][d];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float kv = Ks[tx + 16 * i][d];
+                    acc[0][i] = fmaf(q0, kv, acc[0][i]);
+                    acc[1][i] = fmaf(q1, kv, acc[1][i]);
+                }
+            }
+        }
+        // online softmax over this step's keys
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            float mx = -__builtin_huge_valf();
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = j0 + tx + 16 * i;
+                acc[a][i] = j <= lim[a] ? acc[a][i] * p.scale : -__builtin_huge_valf();
+                mx = fmaxf(mx, acc[a][i]);
+            }
+#pragma unroll
+            for (int of = 8; of > 0; of >>= 1) mx = fmaxf(mx, __shfl_xor(mx, of, 64));
+            const float m_new = fmaxf(m_run[a], mx);
+            const float base = m_new == -__builtin_huge_valf() ? 0.f : m_new;
+            const float f = expf(m_run[a] - base);
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float e = expf(acc[a][i] - base);
+                Ps[2 * ty + a][tx + 16 * i] = e;
+                sum += e;
+            }
+#pragma unroll
+            for (int of = 8; of > 0; of >>= 1) sum += __shfl_xor(sum, of, 64);
+            l_run[a] = l_run[a] * f + sum;
+            m_run[a] = m_new;
+            if (tx == 0) fs[2 * ty + a] = f;
+        }
+        __syncthreads();
+        // O <- O * f + P V
+        const int nk = min(AN, n_keys - j0);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const float f = fs[8 * rg + r];
+#pragma unroll
+            for (int i = 0; i < NC; ++i) o[r][i] *= f;
+        }
+        for (int j = 0; j < nk; ++j) {
+            float vv[NC];
+#pragma unroll
+            for (int i = 0; i < NC; ++i) {
+                const int col = c + 64 * i;
+                vv[i] = col < p.DV ? lda_dt(p.V, p.dt, (vr0 + j0 + j) * p.ldv + (int64_t)head0 * p.v_hs + col) : 0.f;
+            }
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const float pj = Ps[8 * rg + r][j];
+#pragma unroll
+                for (int i = 0; i < NC; ++i) o[r][i] = fmaf(pj, vv[i], o[r][i]);
+            }
+        }
+    }
+    __syncthreads();
+    if (tx == 0) ls[2 * ty] = l_run[0], ls[2 * ty + 1] = l_run[1];
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const int row = 8 * rg + r, tok = tok0 + row / p.hm, head = head0 + row % p.hm;
+        if (tok >= n_new || head >= p.H) continue;
+        const float inv = 1.0f / ls[row];
+        const int64_t ob = (qr0 + tok) * p.ldo + (int64_t)head * p.o_hs;
+#pragma unroll
+        for (int i = 0; i < NC; ++i) {
+            const int col = c + 64 * i;
+            if (col >= p.DV) continue;
+            const float v = o[r][i] * inv;
+            if (p.dt == MI355_DT_F32) ((float*)p.O)[ob + col] = v;
+            else ((bf16_t*)p.O)[ob + col] = f2bf(v);
+        }
+    }
+}
+
+extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, int D2, int DV, const float* Q, int64_t ldq, int q_hs, const void* K1, int64_t ldk1,
+                                 int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
+                                 const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
+                                 int use_mfma, void* stream) {
+    MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && max_new > 0 && H > 0 && D1 > 0 && D2 >= 0 && DV > 0 && DV <= 512 && Q && K1 && V && O && (D2 == 0 || K2),
+                  "latent_attn: bad arguments (value width <= 512)");
+    MI355_REQUIRE(dt == MI355_DT_BF16 || dt == MI355_DT_F32, "latent_attn: bad dtype");
+    MI355_REQUIRE(hm >= 1 && hm <= AM && AM % hm == 0 && (hm == 1 || (k1_hs == 0 && v_hs == 0)), "latent_attn: several heads per tile need shared keys and values (head stride 0)");
+    MI355_REQUIRE(q_row0 && n_new && past && k1_row0 && k2_row0 && v_row0, "latent_attn: sequence descriptors missing");
+    MI355_REQUIRE(ldq >= (int64_t)(H - 1) * q_hs + D1 + D2 && ldo >= (int64_t)(H - 1) * o_hs + DV && ldk1 >= (int64_t)(H - 1) * k1_hs + D1 && ldv >= (int64_t)(H - 1) * v_hs + DV &&
+                      (D2 == 0 || ldk2 >= D2),
+                  "latent_attn: rows too short");
+    LatAttnArgs p;
+    p.Q = Q, p.K1 = K1, p.K2 = K2, p.V = V, p.O = O;
+    p.ldq = ldq, p.ldk1 = ldk1, p.ldk2 = ldk2, p.ldv = ldv, p.ldo = ldo;
+    p.q_hs = q_hs, p.k1_hs = k1_hs, p.v_hs = v_hs, p.o_hs = o_hs;
+    p.D1 = D1, p.D2 = D2, p.DV = DV, p.H = H, p.hm = hm, p.dt = dt;
+    p.q_row0 = q_row0, p.n_new = n_new, p.past = past, p.k1_row0 = k1_row0, p.k2_row0 = k2_row0, p.v_row0 = v_row0;
+    p.scale = scale;
+    const int tm = AM / hm;
+    const int64_t gx = ((int64_t)max_new + tm - 1) / tm, gy = (H + hm - 1) / hm;
+    MI355_REQUIRE(gy <= 65535 && gx < ((int64_t)1 << 31), "latent_attn: grid too large");
+    const dim3 grid((unsigned)gx, (unsigned)gy, n_seq);
+    (void)use_mfma;
+    if (DV <= 64) latent_attn_fma_kernel<1><<<grid, 256, 0, ST(stream)>>>(p);
+    else if (DV <= 128) latent_attn_fma_kernel<2><<<grid, 256, 0, ST(stream)>>>(p);
+    else if (DV <= 256) latent_attn_fma_kernel<4><<<grid, 256, 0, ST(stream)>>>(p);
+    else latent_attn_fma_kernel<8><<<grid, 256, 0, ST(stream)>>>(p);
+    MI355_LAUNCH_CHECK("latent_attn");
+    return 0;
+}

@@ -171,3 +171,107 @@ def generate_batched_loop_kv_cache_left_pad(input_tensor, model, max_gen, contex
     next_pos = attention_mask.sum(dim=-1, keepdim=True)
     return _batched_kv_loop(input_tensor, model, max_gen, context_length, top_k, top_p, min_p, temp, eos_ids, pad_id, device, attention_mask,
                             position_ids, next_pos, lambda lg: lg[:, -1, :])
+
+
+# ----------------------------------------------------------------------------------------------- ragged batches (slot cache, no padding)
+class RaggedBatch:
+    """Scheduler of the serving models of ``registry`` (``model.step`` + ``utils.SlotStateCache``): sequences of different lengths run as ONE packed
+    batch without padding.  A step brings, for every sequence in it, its next tokens -- a whole prompt for a sequence that starts, one token (or more) for
+    one that goes on -- and returns fp32 logits of the rows asked for.  Sequences are named by the caller; ``finish`` gives a sequence's slot back, and
+    the next sequence to start takes it.  A row's logits do not depend on which other sequences share the step."""
+
+    def __init__(self, model, max_tokens=0, slots=4, device=None):
+        self.model = model
+        self.device = device or next(model.parameters()).device
+        self.cache = model.new_cache(self.device, max_tokens=max_tokens, slots=slots)
+
+    def step(self, entries, want=None, return_layers=False):
+        """entries: [(seq_id, [token, ...])] in batch order.  want: per entry the positions among ITS new tokens whose logits are asked for (default:
+        the last one).  Returns fp32 [rows asked for, vocab] in the order of the entries and of ``want`` (None if nothing is asked for)."""
+        from .common.mixers import SeqStep
+
+        if not entries:
+            return None
+        cache, vocab = self.cache, self.model.vocab_size
+        slotted = []
+        for seq_id, toks in entries:
+            toks = [int(t) for t in toks]
+            if any(t < 0 or t >= vocab for t in toks):
+                raise ValueError(f"sequence {seq_id!r}: token id outside [0, {vocab})")
+            slot = cache.slot(seq_id) if seq_id in cache else cache.open(seq_id)
+            slotted.append((slot, toks))
+        st = SeqStep(cache, slotted, self.device, self.model.act_dtype)
+        rows = []
+        for i, (_, toks) in enumerate(slotted):
+            w = [len(toks) - 1] if want is None else want[i]
+            for p in w:
+                if not 0 <= p < len(toks):
+                    raise ValueError("a wanted position lies outside the entry's tokens")
+                rows.append(st.host_seq_off[i] + p)
+        # the whole stack runs even when no logits are asked for: the step still has to leave its rows and state behind
+        want_rows = torch.tensor(rows if rows else [0], dtype=torch.long).to(self.device)
+        out = self.model.step(st, want_rows, return_layers=return_layers)
+        for slot, toks in slotted:
+            cache.advance(slot, toks)
+        if return_layers:
+            return (out[0] if rows else None), out[1]
+        return out if rows else None
+
+    def finish(self, seq_id):
+        self.cache.close(seq_id)
+
+
+def generate_ragged(model, prompts, max_gen, top_k=None, top_p=None, min_p=None, temp=0.0, eos_ids=None, max_tokens=0):
+    """Generation for a list of prompts of different lengths (lists of token ids) through ``RaggedBatch``: all prompts start together in one packed
+    step, then every unfinished sequence goes on by one sampled token per step; a sequence that produced an eos id (or ``max_gen`` tokens) leaves the
+    batch and frees its slot.  Returns the generated ids per prompt (eos not included)."""
+    eos = set(eos_ids if isinstance(eos_ids, (list, tuple, set)) else ([] if eos_ids is None else [eos_ids]))
+    batch = RaggedBatch(model, max_tokens=max_tokens, slots=max(1, len(prompts)))
+    out = [[] for _ in prompts]
+    live = list(range(len(prompts)))
+    entries = [(i, list(prompts[i])) for i in live]
+    for _ in range(max_gen):
+        if not entries:
+            break
+        logits = batch.step(entries)
+        nxt = sampling(logits, top_k, top_p, min_p, temp).view(-1).tolist()
+        entries, still = [], []
+        for i, t in zip(live, nxt):
+            if t in eos:
+                batch.finish(i)
+                continue
+            out[i].append(int(t))
+            if len(out[i]) >= max_gen:
+                batch.finish(i)
+                continue
+            entries.append((i, [int(t)]))
+            still.append(i)
+        live = still
+    return out
+
+
+def main(argv=None):
+    """``python -m llm_quest_amd.generate --model DIR --prompt 5,17,3 --prompt 9,2 --max-gen 16``: greedy or sampled continuation of token-id prompts
+    with a serving model chosen by the folder's config.json."""
+    import argparse
+    import json
+
+    from . import registry
+
+    ap = argparse.ArgumentParser(description="generate token ids with a serving model (ragged batch, slot cache)")
+    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--dtype", default="bfloat16", choices=sorted(registry.DTYPES))
+    ap.add_argument("--prompt", action="append", required=True, help="comma-separated token ids; repeat for a batch")
+    ap.add_argument("--max-gen", type=int, default=16)
+    ap.add_argument("--temp", type=float, default=0.0)
+    ap.add_argument("--top-k", type=int, default=None)
+    ap.add_argument("--top-p", type=float, default=None)
+    ap.add_argument("--eos", type=int, action="append", default=None)
+    a = ap.parse_args(argv)
+    model = registry.load_model(a.model, a.dtype, "cuda")
+    prompts = [[int(t) for t in p.split(",") if t.strip()] for p in a.prompt]
+    print(json.dumps(generate_ragged(model, prompts, a.max_gen, top_k=a.top_k, top_p=a.top_p, temp=a.temp, eos_ids=a.eos)))
+
+
+if __name__ == "__main__":
+    main()

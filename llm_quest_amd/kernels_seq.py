@@ -1,0 +1,204 @@
+"""Python launchers of the ragged-batch serving kernels (csrc/seqmix.hip, csrc/bgemm.hip, csrc/latent_attn.hip): hashed-bigram embedding,
+post-sum LayerNorm on an fp32 residual stream, latent key/value rows, interleaved rotary embedding, two-part-key attention, gated linear
+attention with carried state, the grouped sigmoid router and the grouped expert products.
+
+Activations are bf16 (serving mode: bf16 operands, fp32 accumulation) or fp32 (true 32-bit mode: every product is an fp32 FMA chain; the bf16
+weights are exactly representable and widened on load).  Whatever the mode, the residual stream, norm statistics, rotary angles, decays,
+recurrent state and the router are fp32.  There is no CPU path.
+"""
+
+import torch
+
+from . import _lib as L
+from . import kernels as K
+
+BF16, F32, I32 = torch.bfloat16, torch.float32, torch.int32
+
+
+def _dt(t):
+    return L.dt_code(t.dtype)
+
+
+def _rows(t, name):
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError(f"{name}: a 2-D tensor with unit inner stride is required, got shape {tuple(t.shape)} strides {t.stride()}")
+
+
+def _i32(t, name, n=None):
+    if t.dtype != I32 or not t.is_contiguous() or (n is not None and t.numel() < n):
+        raise ValueError(f"{name}: contiguous int32 tensor{'' if n is None else f' of at least {n} entries'} required")
+
+
+def embed_hash(tok, prev, table, scale, bigram=None, buckets=0, mul_prev=0, mul_cur=0):
+    """fp32 [tokens, width] = table[tok] * scale (+ bigram row hashed from (prev, tok); prev < 0 selects row ``buckets``)."""
+    L.require_gpu(tok, prev, table, bigram)
+    T = tok.numel()
+    _i32(tok, "embed_hash(tok)")
+    if bigram is not None:
+        _i32(prev, "embed_hash(prev)", T)
+        if bigram.dtype != BF16 or not bigram.is_contiguous() or tuple(bigram.shape) != (buckets + 1, table.shape[1]):
+            raise ValueError("embed_hash: the bigram table is bf16 [buckets + 1, width]")
+    if table.dtype != BF16 or not table.is_contiguous():
+        raise ValueError("embed_hash: the table is contiguous bf16")
+    out = torch.empty((T, table.shape[1]), dtype=F32, device=table.device)
+    L.call("mi355_embed_hash_fwd", T, table.shape[1], table.shape[0], L.ptr(tok), L.ptr(prev), L.ptr(table), float(scale), L.ptr(bigram), int(buckets),
+           int(mul_prev), int(mul_cur), L.ptr(out))
+    return out
+
+
+def add_layernorm(x, w, b, eps, alpha=1.0, y=None, parts=1, cast_dtype=None):
+    """LayerNorm(alpha * x + sum of y's ``parts`` rows per token) on fp32 rows -> (fp32 rows, the same rows in ``cast_dtype`` or None)."""
+    L.require_gpu(x, w, b, y)
+    _rows(x, "add_layernorm(x)")
+    T, width = x.shape
+    if x.dtype != F32 or not x.is_contiguous() or w.dtype != F32 or b.dtype != F32 or w.numel() != width or b.numel() != width:
+        raise ValueError("add_layernorm: x contiguous fp32 [tokens, width], weight and bias fp32 [width]")
+    if y is not None:
+        _rows(y, "add_layernorm(y)")
+        if y.shape[0] != T * parts or y.shape[1] != width:
+            raise ValueError(f"add_layernorm: the summand must be [{T * parts}, {width}], got {tuple(y.shape)}")
+    out = torch.empty_like(x)
+    cast = None if cast_dtype is None or cast_dtype == F32 else torch.empty((T, width), dtype=cast_dtype, device=x.device)
+    L.call("mi355_add_layernorm_fwd", T, width, L.ptr(x), float(alpha), L.ptr(y), 0 if y is None else _dt(y), 0 if y is None else y.stride(0), int(parts),
+           L.ptr(w), L.ptr(b), float(eps), L.ptr(out), L.ptr(cast), 0 if cast is None else _dt(cast))
+    return out, (out if cast_dtype == F32 else cast)
+
+
+def rmsnorm_rows(x, w, eps, out_dtype=None):
+    L.require_gpu(x, w)
+    _rows(x, "rmsnorm_rows(x)")
+    if w.dtype != F32 or w.numel() != x.shape[1]:
+        raise ValueError("rmsnorm_rows: weight fp32 [n]")
+    out = torch.empty(x.shape, dtype=out_dtype or x.dtype, device=x.device)
+    L.call("mi355_rmsnorm_rows", x.shape[0], x.shape[1], L.ptr(x), _dt(x), x.stride(0), L.ptr(w), float(eps), L.ptr(out), _dt(out), out.stride(0))
+    return out
+
+
+def rope_frequencies(dims, base, device):
+    """fp32 [dims / 2]: base^(-2i / dims), evaluated in double."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).to(F32).to(device)
+
+
+def latent_kv_append(src, rank, rot, w, eps, pos, dst_row, freq, dims, cache2d):
+    """src [tokens, rank + rot] -> rows ``dst_row`` of ``cache2d`` [rows, rank + rot]: RMSNorm on the latent, interleaved rotary on the shared key part."""
+    L.require_gpu(src, w, pos, dst_row, freq, cache2d)
+    _rows(src, "latent_kv_append(src)")
+    _rows(cache2d, "latent_kv_append(cache)")
+    T = src.shape[0]
+    _i32(pos, "latent_kv_append(pos)", T)
+    _i32(dst_row, "latent_kv_append(dst_row)", T)
+    if src.shape[1] != rank + rot or cache2d.shape[1] != rank + rot or w.dtype != F32 or w.numel() != rank or (dims and (freq.dtype != F32 or freq.numel() < dims // 2)):
+        raise ValueError("latent_kv_append: operand sizes do not match rank / rot")
+    L.call("mi355_latent_kv_append", T, rank, rot, L.ptr(src), _dt(src), src.stride(0), L.ptr(w), float(eps), L.ptr(pos), L.ptr(dst_row), L.ptr(freq), int(dims),
+           L.ptr(cache2d), _dt(cache2d), cache2d.stride(0))
+
+
+def rope_heads(src, H, n, src_hs, src_off, dst, dst_hs, dst_off, rot_start, dims, freq, pos):
+    """dst (fp32) <- n entries per head of src, the pairs of [rot_start, rot_start + dims) rotated by the token's position."""
+    L.require_gpu(src, dst, freq, pos)
+    _rows(src, "rope_heads(src)")
+    _rows(dst, "rope_heads(dst)")
+    if dst.dtype != F32 or dst.shape[0] != src.shape[0]:
+        raise ValueError("rope_heads: dst is fp32 with src's rows")
+    _i32(pos, "rope_heads(pos)", src.shape[0])
+    if src.shape[1] < (H - 1) * src_hs + src_off + n or dst.shape[1] < (H - 1) * dst_hs + dst_off + n:
+        raise ValueError("rope_heads: rows too short for the head layout")
+    L.call("mi355_rope_heads", src.shape[0], H, n, L.ptr(src), _dt(src), src.stride(0), src_hs, src_off, L.ptr(dst), dst.stride(0), dst_hs, dst_off, rot_start, dims,
+           L.ptr(freq), L.ptr(pos))
+    return dst
+
+
+def gated_headnorm(o, w, gate, H, D, eps, out_dtype):
+    L.require_gpu(o, w, gate)
+    _rows(gate, "gated_headnorm(gate)")
+    if o.dtype != F32 or not o.is_contiguous() or o.shape[1] != H * D or gate.shape != o.shape or w.dtype != F32 or w.numel() != D:
+        raise ValueError("gated_headnorm: o contiguous fp32 [tokens, H*D], gate a view of that shape, weight fp32 [D]")
+    out = torch.empty(o.shape, dtype=out_dtype, device=o.device)
+    L.call("mi355_gated_headnorm", o.shape[0], H, D, L.ptr(o), L.ptr(w), L.ptr(gate), _dt(gate), gate.stride(0), float(eps), L.ptr(out), _dt(out), out.stride(0))
+    return out
+
+
+def gla(q, k, v, z, zbias, inv_tau, qscale, seq_off, slot, state, H, dk, dv):
+    """Gated linear attention over a ragged batch; ``state`` fp32 [slots, H, dk, dv] is read and written at ``slot``.  Returns fp32 [tokens, H * dv]."""
+    L.require_gpu(q, k, v, z, zbias, seq_off, slot, state)
+    for t, n, w in ((q, "q", H * dk), (k, "k", H * dk), (z, "z", H * dk), (v, "v", H * dv)):
+        _rows(t, f"gla({n})")
+        if t.shape[1] != w or (n != "z" and t.dtype != q.dtype) or t.shape[0] != q.shape[0]:
+            raise ValueError(f"gla({n}): [tokens, {w}] of q's dtype required")
+    n_seq = slot.numel()
+    _i32(seq_off, "gla(seq_off)", n_seq + 1)
+    _i32(slot, "gla(slot)")
+    if state.dtype != F32 or not state.is_contiguous() or tuple(state.shape[1:]) != (H, dk, dv) or zbias.dtype != F32 or zbias.numel() != H * dk:
+        raise ValueError("gla: state fp32 [slots, H, dk, dv], bias fp32 [H * dk]")
+    o = torch.empty((q.shape[0], H * dv), dtype=F32, device=q.device)
+    L.call("mi355_gla_fwd", n_seq, L.ptr(seq_off), L.ptr(slot), H, dk, dv, L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(z), _dt(q), _dt(z), q.stride(0), k.stride(0), v.stride(0),
+           z.stride(0), L.ptr(zbias), float(inv_tau), float(qscale), L.ptr(state), L.ptr(o))
+    return o
+
+
+def moe_route(logits, correction, top, groups, keep, scale):
+    L.require_gpu(logits, correction)
+    if logits.dtype != F32 or not logits.is_contiguous() or (correction is not None and (correction.dtype != F32 or correction.numel() != logits.shape[1])):
+        raise ValueError("moe_route: logits contiguous fp32 [tokens, experts], correction fp32 [experts]")
+    T, E = logits.shape
+    ids = torch.empty((T, top), dtype=I32, device=logits.device)
+    wts = torch.empty((T, top), dtype=F32, device=logits.device)
+    L.call("mi355_moe_route", T, E, top, groups, keep, L.ptr(logits), L.ptr(correction), float(scale), L.ptr(ids), L.ptr(wts))
+    return ids, wts
+
+
+def moe_dispatch(ids, E):
+    L.require_gpu(ids)
+    _i32(ids, "moe_dispatch(ids)")
+    offs = torch.empty((E + 1,), dtype=I32, device=ids.device)
+    perm = torch.empty((ids.numel(),), dtype=I32, device=ids.device)
+    L.call("mi355_moe_dispatch", ids.numel(), E, L.ptr(ids), L.ptr(offs), L.ptr(perm))
+    return offs, perm
+
+
+def bgemm(a, b, c, M, N, Kd, batch=1, lda=None, a_bs=0, sbn=None, sbk=1, b_bs=0, ldc=None, c_bs=0, grp_offs=None, a_rows=None, a_div=1, c_rows=None,
+          row_scale=None, epi=0, mfma=None):
+    """The general strided product (see include/mi355_vlm.h).  Strides default to a's / c's row pitch and b stored [N, K]; the caller vouches that the
+    strides stay inside the tensors.  ``mfma`` defaults to bf16 a and b."""
+    L.require_gpu(a, b, c, grp_offs, a_rows, c_rows, row_scale)
+    if mfma is None:
+        mfma = a.dtype == BF16 and b.dtype == BF16
+    L.call("mi355_bgemm", batch, M, N, Kd, L.ptr(a), _dt(a), a.stride(0) if lda is None else lda, a_bs, L.ptr(b), _dt(b), b.stride(0) if sbn is None else sbn, sbk, b_bs,
+           L.ptr(c), _dt(c), c.stride(0) if ldc is None else ldc, c_bs, L.ptr(grp_offs), L.ptr(a_rows), a_div, L.ptr(c_rows), L.ptr(row_scale), epi, 1 if mfma else 0)
+    return c
+
+
+def linear(x, w, out_dtype=None):
+    """x [M, K] (bf16 or fp32) times w[N, K]^T (bf16).  bf16 rows go through the MFMA GEMMs (weight stream for <= 8 rows), fp32 rows through the fp32 FMA product."""
+    _rows(x, "linear(x)")
+    M, Kd = x.shape
+    N = w.shape[0]
+    if w.dtype != BF16 or w.shape[1] != Kd or w.stride(1) != 1:
+        raise ValueError("linear: weight bf16 [N, K] with unit inner stride")
+    out_dtype = out_dtype or x.dtype
+    if x.dtype == BF16:
+        aligned = Kd % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+        if aligned and M <= 8 and out_dtype == BF16:
+            from . import ops_decode
+
+            return ops_decode.gemv(x, w)
+        if aligned and M > 8:
+            return K.gemm(L.GEMM_NT, x, w, out_dtype=out_dtype)
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    return bgemm(x, w, out, M, N, Kd)
+
+
+def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, desc, max_new, scale):
+    """Two-part-key causal attention over a ragged batch.  ``desc`` = (q_row0, n_new, past, k1_row0, k2_row0, v_row0) int32 [n_seq] each."""
+    L.require_gpu(q, k1, k2, v, out, *desc)
+    for t, n in ((q, "q"), (k1, "k1"), (v, "v"), (out, "out")):
+        _rows(t, f"latent_attn({n})")
+    if q.dtype != F32 or k1.dtype != v.dtype or out.dtype != v.dtype or (k2 is not None and k2.dtype != v.dtype):
+        raise ValueError("latent_attn: q fp32; keys, values and output share one dtype")
+    n_seq = desc[0].numel()
+    for t in desc:
+        _i32(t, "latent_attn(desc)", n_seq)
+    L.call("mi355_latent_attn", n_seq, max_new, H, hm, D1, D2, DV, L.ptr(q), q.stride(0), q_hs, L.ptr(k1), k1.stride(0), k1_hs, L.ptr(k2), 0 if k2 is None else k2.stride(0),
+           L.ptr(v), v.stride(0), v_hs, L.ptr(out), out.stride(0), o_hs, _dt(v), *[L.ptr(t) for t in desc], float(scale), 1 if v.dtype == BF16 else 0)
+    return out

@@ -138,6 +138,128 @@ class Qwen3_5Cache:
         self.recurrent_states[layer_idx] = recurrent_state
 
 
+class SlotStateCache:
+    """Per-sequence state of hybrid decoders served in RAGGED batches (no padding): every live sequence owns a slot.
+
+    Where ``KVCache`` keeps one ``[batch, capacity, width]`` buffer per layer for a batch that advances in lockstep, here each sequence has its own
+    length, sequences join and leave, and a slot is reused by the next sequence.  Per layer, by ``layer_specs[i]``:
+      * ``("rows", width)``  -- token-major rows ``[slots, capacity, width]`` in the activation dtype (the latent + rotated-key rows of latent attention);
+        row ``slot * capacity + position`` of the 2-D view ``rows2d(i)`` is what the kernels address;
+      * ``("shared", j)``    -- the layer reads layer j's rows and stores nothing;
+      * ``("state", shape)`` -- a fixed-size fp32 state ``[slots, *shape]`` (the matrix state of linear attention), zeroed when a slot is opened;
+      * ``None``             -- nothing.
+    Besides, per slot: the length so far and the last token (the embedding of some designs looks one token back).  Growth follows ``KVCache``: the row
+    capacity starts at what the first sequences need plus ``initial_chunk_size`` and grows by whole ``chunk_size`` steps up to ``context_len``; slots double."""
+
+    def __init__(self, layer_specs, context_len, device, dtype, slots=4, capacity=0, initial_chunk_size=512, chunk_size=256):
+        self.layer_specs = list(layer_specs)
+        self.context_len = int(context_len)
+        self.device, self.dtype = device, dtype
+        self.chunk_size, self.initial_chunk_size = chunk_size, initial_chunk_size
+        self.slots = max(1, int(slots))
+        self.capacity = min(self.context_len, int(capacity))
+        self.rows = [None] * len(self.layer_specs)
+        self.states = [None] * len(self.layer_specs)
+        self.length = [0] * self.slots
+        self.last_token = [-1] * self.slots
+        self._slot_of = {}
+        self._free = list(range(self.slots))
+        self.reuses = 0  # slots handed out again after a close (bookkeeping for tests / logs)
+        self._used_once = set()
+        for i, spec in enumerate(self.layer_specs):
+            if spec is not None and spec[0] == "state":
+                self.states[i] = torch.zeros((self.slots,) + tuple(spec[1]), dtype=torch.float32, device=device)
+        if self.capacity:
+            self._allocate_rows(self.capacity)
+
+    # ------------------------------------------------------------------ storage
+    def _allocate_rows(self, capacity):
+        for i, spec in enumerate(self.layer_specs):
+            if spec is None or spec[0] != "rows":
+                continue
+            old = self.rows[i]
+            new = torch.zeros((self.slots, capacity, spec[1]), dtype=self.dtype, device=self.device)
+            if old is not None:
+                n = min(old.shape[0], self.slots)
+                new[:n, : old.shape[1]].copy_(old[:n])
+            self.rows[i] = new
+        self.capacity = capacity
+
+    def _grow_slots(self):
+        add = self.slots
+        self._free.extend(range(self.slots, self.slots + add))
+        self.slots += add
+        self.length.extend([0] * add)
+        self.last_token.extend([-1] * add)
+        for i, st in enumerate(self.states):
+            if st is not None:
+                self.states[i] = torch.cat([st, torch.zeros_like(st)], dim=0)
+        if self.capacity:
+            self._allocate_rows(self.capacity)
+
+    def reserve(self, needed):
+        """Make room for sequences of up to ``needed`` tokens (contents kept)."""
+        if needed > self.context_len:
+            raise ValueError(f"SlotStateCache: {needed} tokens exceed context_len {self.context_len}")
+        if needed <= self.capacity:
+            return
+        if self.capacity == 0:
+            cap = needed + self.initial_chunk_size
+        else:
+            cap = self.capacity + -(-(needed - self.capacity) // self.chunk_size) * self.chunk_size
+        self._allocate_rows(min(cap, self.context_len))
+
+    # ------------------------------------------------------------------ sequences
+    def open(self, seq_id):
+        """A slot for a new sequence: length 0, no last token, zero state."""
+        if seq_id in self._slot_of:
+            raise KeyError(f"SlotStateCache: sequence {seq_id!r} is already open")
+        if not self._free:
+            self._grow_slots()
+        self._free.sort()
+        slot = self._free.pop(0)
+        if slot in self._used_once:
+            self.reuses += 1
+        self._used_once.add(slot)
+        self._slot_of[seq_id] = slot
+        self.length[slot] = 0
+        self.last_token[slot] = -1
+        for st in self.states:
+            if st is not None:
+                st[slot].zero_()
+        return slot
+
+    def slot(self, seq_id):
+        return self._slot_of[seq_id]
+
+    def __contains__(self, seq_id):
+        return seq_id in self._slot_of
+
+    def close(self, seq_id):
+        """Give the sequence's slot back; its rows and state are dead from now on."""
+        self._free.append(self._slot_of.pop(seq_id))
+
+    @property
+    def live_tokens(self):
+        return sum(self.length[s] for s in self._slot_of.values())
+
+    def advance(self, slot, tokens):
+        self.length[slot] += len(tokens)
+        self.last_token[slot] = int(tokens[-1])
+
+    # ------------------------------------------------------------------ views for the kernels
+    def source(self, layer_idx):
+        spec = self.layer_specs[layer_idx]
+        return spec[1] if spec is not None and spec[0] == "shared" else layer_idx
+
+    def rows2d(self, layer_idx):
+        r = self.rows[self.source(layer_idx)]
+        return r.view(r.shape[0] * r.shape[1], r.shape[2])
+
+    def state(self, layer_idx):
+        return self.states[layer_idx]
+
+
 # ----------------------------------------------------------------------------------------------- checkpoint import (row f2)
 # API of the "WEIGHTS LOADING" helpers of llm_quest/utils.py:921-1035.  The build / GPU boxes have no network, so
 # ``download_hf_weights`` resolves its argument against the local filesystem (a .safetensors file, a directory of shards with
