@@ -448,6 +448,8 @@ int mi355_kv_append(int B, int width, const void* k_rows, int64_t ldk, const voi
 /* Greedy sampling (generate.py:472-476, temp == 0): out[r] = index of the row maximum of bf16 logits [rows, V] (first on ties).
  * workspace: rows * 64 * 12 bytes (+8), 8-byte aligned: 64 column ranges per row are scanned in parallel, then merged. */
 int mi355_argmax_rows(int64_t rows, int64_t V, const void* logits, int64_t ld, int64_t* out, void* workspace, void* stream);
+/* The same on fp32 logits (the serving models return fp32 logits). */
+int mi355_argmax_rows_f32(int64_t rows, int64_t V, const float* logits, int64_t ld, int64_t* out, void* workspace, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------------
  * Measurement aid (csrc/probe.hip), no reference counterpart: `blocks` workgroups of four waves run reps x 16 v_mfma_f32_32x32x16_bf16 on random

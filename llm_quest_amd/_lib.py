@@ -99,6 +99,7 @@ SIGNATURES = {
     "mi355_attn_decode": [_I, _I, _I, _I, _P, _P, _P, _L, _L, _I, _P, _P, _L, _P, _F, _I, _P, _P],
     "mi355_kv_append": [_I, _I, _P, _L, _P, _L, _P, _P, _L, _L, _I, _P, _P],
     "mi355_argmax_rows": [_L, _L, _P, _L, _P, _P, _P],
+    "mi355_argmax_rows_f32": [_L, _L, _P, _L, _P, _P, _P],
     # ragged-batch serving of hybrid decoders (csrc/seqmix.hip, csrc/bgemm.hip, csrc/latent_attn.hip)
     "mi355_embed_hash_fwd": [_L, _I, _I, _P, _P, _P, _F, _P, _I, _I, _I, _P, _P],
     "mi355_add_layernorm_fwd": [_L, _I, _P, _F, _P, _I, _L, _I, _P, _P, _F, _P, _P, _I, _P],

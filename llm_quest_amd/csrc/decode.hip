@@ -467,15 +467,18 @@ __device__ __forceinline__ void argmax_merge(float& best, int64_t& idx, float ov
         idx = oi;
     }
 }
-__global__ __launch_bounds__(256) void argmax_part_kernel(int64_t V, const bf16_t* __restrict__ x, int64_t ld, float* __restrict__ pv, int64_t* __restrict__ pi) {
+__device__ __forceinline__ float argmax_load(const bf16_t* p) { return bf2f(*p); }
+__device__ __forceinline__ float argmax_load(const float* p) { return *p; }
+template <typename T>
+__global__ __launch_bounds__(256) void argmax_part_kernel(int64_t V, const T* __restrict__ x, int64_t ld, float* __restrict__ pv, int64_t* __restrict__ pi) {
     __shared__ float bv[4];
     __shared__ int64_t bi[4];
-    const bf16_t* r = x + (int64_t)blockIdx.y * ld;
+    const T* r = x + (int64_t)blockIdx.y * ld;
     const int64_t span = (V + ARG_SPLIT - 1) / ARG_SPLIT, c0 = blockIdx.x * span, c1 = c0 + span < V ? c0 + span : V;
     float best = -__builtin_huge_valf();
     int64_t idx = 0x7fffffffffffffffll;
     for (int64_t i = c0 + threadIdx.x; i < c1; i += 256) {
-        const float v = bf2f(r[i]);
+        const float v = argmax_load(r + i);
         if (v > best) {
             best = v;
             idx = i;
@@ -601,9 +604,20 @@ extern "C" int mi355_argmax_rows(int64_t rows, int64_t V, const void* logits, in
     static_assert(ARG_SPLIT == 64, "the merge kernel is one wave");
     float* pv = (float*)workspace;
     int64_t* pi = (int64_t*)((char*)workspace + ((rows * ARG_SPLIT * 4 + 7) / 8) * 8);
-    argmax_part_kernel<<<dim3(ARG_SPLIT, (unsigned)rows), 256, 0, ST(stream)>>>(V, (const bf16_t*)logits, ld, pv, pi);
+    argmax_part_kernel<bf16_t><<<dim3(ARG_SPLIT, (unsigned)rows), 256, 0, ST(stream)>>>(V, (const bf16_t*)logits, ld, pv, pi);
     MI355_LAUNCH_CHECK("argmax_rows(part)");
     argmax_merge_kernel<<<(int)rows, 64, 0, ST(stream)>>>(pv, pi, out);
     MI355_LAUNCH_CHECK("argmax_rows");
+    return 0;
+}
+
+extern "C" int mi355_argmax_rows_f32(int64_t rows, int64_t V, const float* logits, int64_t ld, int64_t* out, void* workspace, void* stream) {
+    MI355_REQUIRE(rows > 0 && rows <= 65535 && V > 0 && logits && out && workspace && ld >= V, "argmax_rows_f32: bad arguments (workspace: rows * 64 * 12 bytes)");
+    float* pv = (float*)workspace;
+    int64_t* pi = (int64_t*)((char*)workspace + ((rows * ARG_SPLIT * 4 + 7) / 8) * 8);
+    argmax_part_kernel<float><<<dim3(ARG_SPLIT, (unsigned)rows), 256, 0, ST(stream)>>>(V, logits, ld, pv, pi);
+    MI355_LAUNCH_CHECK("argmax_rows_f32(part)");
+    argmax_merge_kernel<<<(int)rows, 64, 0, ST(stream)>>>(pv, pi, out);
+    MI355_LAUNCH_CHECK("argmax_rows_f32");
     return 0;
 }

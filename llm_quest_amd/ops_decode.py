@@ -120,11 +120,11 @@ def attn_decode(q, kc, vc, length, Hq, Hkv, D, key_mask=None, scale=None, len_de
 
 def argmax_rows(logits2d):
     L.require_gpu(logits2d)
-    if logits2d.dtype != BF16 or logits2d.dim() != 2 or logits2d.stride(1) != 1:
-        raise ValueError("argmax_rows: bf16 [rows, V] with unit inner stride")
+    if logits2d.dtype not in (BF16, torch.float32) or logits2d.dim() != 2 or logits2d.stride(1) != 1:
+        raise ValueError("argmax_rows: bf16 or fp32 [rows, V] with unit inner stride")
     out = torch.empty(logits2d.shape[0], dtype=torch.int64, device=logits2d.device)
     ws = torch.empty(logits2d.shape[0] * 64 * 12 // 8 + 2, dtype=torch.int64, device=logits2d.device)
-    L.call("mi355_argmax_rows", logits2d.shape[0], logits2d.shape[1], L.ptr(logits2d), logits2d.stride(0), L.ptr(out), L.ptr(ws))
+    L.call("mi355_argmax_rows" if logits2d.dtype == BF16 else "mi355_argmax_rows_f32", logits2d.shape[0], logits2d.shape[1], L.ptr(logits2d), logits2d.stride(0), L.ptr(out), L.ptr(ws))
     return out
 
 

@@ -1,0 +1,424 @@
+"""GPU tests of the Gemepel serving path against the plain oracle (oracle/gemepel.py): each mechanism's kernel alone, then the model through the
+registry, the slot cache and the ragged-batch scheduler -- whole prompts, token-by-token decoding, portions, unequal batches, reused slots, far keys,
+odd sizes, greedy generation.  fp32 mode is held to fp32 rounding; bf16 mode to a few bf16 roundings of the logits' scale."""
+
+import json
+import math
+
+import pytest
+import torch
+
+from oracle import gemepel as G
+from tests import gemepel_util as U
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
+
+
+def dev_i32(x):
+    return torch.tensor(x, dtype=I32).to(DEV)
+
+
+def rel(a, b):
+    a, b = a.detach().float().cpu(), b.detach().float().cpu()
+    return float((a - b).norm() / (b.norm() + 1e-30))
+
+
+def row_err(got, want, quantile=None):
+    """Per row: rms of the difference (mean removed) over the rms of the wanted rows; the worst row, or a quantile of the rows.
+
+    bf16 runs of whole models are judged on the median row: with random weights and a dozen experts a good part of the tokens has two choice scores
+    within a bf16 rounding of the residual stream, and the other expert is then a legitimate choice that moves that token's row.  The fp32 runs, and
+    the bf16 runs of every kernel alone, are judged on every row."""
+    got, want = got.detach().float().cpu(), want.detach().float().cpu()
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    e = d.pow(2).mean(-1).sqrt() / want.pow(2).mean().sqrt()
+    return e.max().item() if quantile is None else torch.quantile(e, quantile).item()
+
+
+def model_err(got, want, dt):
+    return row_err(got, want, None if dt == "float32" else 0.5)
+
+
+TOL = {"float32": 2e-5, "bfloat16": 6e-2}
+
+
+# ------------------------------------------------------------------------------------------------------------------- models through the registry
+@pytest.fixture(scope="module")
+def checkpoint(tmp_path_factory):
+    cfg = U.make_config(U.default_layers())
+    w = U.make_weights(cfg, 11)
+    return U.save(str(tmp_path_factory.mktemp("gemepel")), cfg, w), cfg, w
+
+
+@pytest.fixture(scope="module")
+def models(checkpoint):
+    from llm_quest_amd import registry
+
+    folder, cfg, w = checkpoint
+    return {dt: registry.load_model(folder, dt, DEV) for dt in ("float32", "bfloat16")}, cfg, w
+
+
+def tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+_oracle_cache = {}
+
+
+def oracle(cfg, w, toks, layers=False):
+    key = (id(w), tuple(toks), layers)
+    if key not in _oracle_cache:
+        _oracle_cache[key] = G.forward(toks, w, cfg, torch.float32, return_layers=layers)
+    return _oracle_cache[key]
+
+
+def batch_of(model, **kw):
+    from llm_quest_amd.generate import RaggedBatch
+
+    return RaggedBatch(model, **kw)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_whole_prompt_every_layer(models, dt):
+    ms, cfg, w = models
+    toks = tokens(70, cfg["vocab"], 1)
+    want, layers = oracle(cfg, w, toks, layers=True)
+    b = batch_of(ms[dt])
+    got, got_layers = b.step([("a", toks)], [list(range(len(toks)))], return_layers=True)
+    for i, l in enumerate(got_layers):
+        assert model_err(l, layers[i], dt) < (2e-5 if dt == "float32" else 8e-2), f"residual stream after layer {i}"
+    assert model_err(got, want, dt) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_token_by_token_from_the_first_token(models, dt):
+    """Every token alone: the first one starts the sequence (bigram row of a sequence start, empty state), all others run the continuation path."""
+    ms, cfg, w = models
+    toks = tokens(45, cfg["vocab"], 2)
+    want = oracle(cfg, w, toks)
+    b = batch_of(ms[dt])
+    got = torch.cat([b.step([("a", [t])]) for t in toks])
+    assert model_err(got, want, dt) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_portions_of_several_sizes(models, dt):
+    ms, cfg, w = models
+    toks = tokens(90, cfg["vocab"], 3)
+    want = oracle(cfg, w, toks)
+    b = batch_of(ms[dt])
+    got, at = [], 0
+    for n in [7, 2, 2, 33, 1, 9, 2, 34]:
+        got.append(b.step([("a", toks[at : at + n])], [list(range(n))]))
+        at += n
+    assert at == len(toks)
+    assert model_err(torch.cat(got), want, dt) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_unequal_batch_equals_each_request_alone(models, dt):
+    ms, cfg, w = models
+    lens, tail = [3, 41, 17, 66], 9
+    seqs = [tokens(n + tail, cfg["vocab"], 10 + i) for i, n in enumerate(lens)]
+    alone = []
+    for s in seqs:
+        b = batch_of(ms[dt])
+        alone.append(b.step([("x", s)], [list(range(len(s)))]))
+    b = batch_of(ms[dt], slots=2)  # fewer slots than sequences: the cache grows
+    got = [[] for _ in seqs]
+    out = b.step([(i, s[: lens[i]]) for i, s in enumerate(seqs)], [list(range(n)) for n in lens])
+    at = 0
+    for i, n in enumerate(lens):
+        got[i].append(out[at : at + n])
+        at += n
+    live = list(range(len(seqs)))
+    for k in range(tail):
+        if k == 4:  # two requests leave early; the others go on
+            for i in (0, 2):
+                b.finish(i)
+                live.remove(i)
+        out = b.step([(i, [seqs[i][lens[i] + k]]) for i in live])
+        for j, i in enumerate(live):
+            got[i].append(out[j : j + 1])
+    for i, s in enumerate(seqs):
+        g = torch.cat(got[i])
+        ref = alone[i][: g.shape[0]]
+        assert model_err(g, ref, dt) < (1e-5 if dt == "float32" else 3e-2), f"request {i} in the batch differs from the request alone"
+        assert model_err(g, oracle(cfg, w, s)[: g.shape[0]], dt) < TOL[dt]
+
+
+def test_freed_slots_are_reused_without_leftovers(models):
+    """A long sequence leaves rows and state behind; the next, shorter one takes its slot and must not see any of it.  The cache starts small, so the
+    rows also grow while a sequence is alive."""
+    ms, cfg, w = models
+    b = batch_of(ms["float32"], slots=1)
+    b.cache.initial_chunk_size, b.cache.chunk_size = 4, 8
+    long_, short = tokens(60, cfg["vocab"], 20), tokens(21, cfg["vocab"], 21)
+    b.step([("long", long_[:50])])
+    for t in long_[50:]:
+        b.step([("long", [t])])
+    b.finish("long")
+    got = [b.step([("short", short[:12])], [list(range(12))])] + [b.step([("short", [t])]) for t in short[12:]]
+    assert b.cache.reuses >= 1 and b.cache.slots == 1
+    assert row_err(torch.cat(got), oracle(cfg, w, short)) < TOL["float32"]
+
+
+def test_long_decoding(models):
+    ms, cfg, w = models
+    toks = tokens(260, cfg["vocab"], 30)
+    b = batch_of(ms["float32"])
+    b.step([("a", toks[:5])])
+    got = torch.cat([b.step([("a", [t])]) for t in toks[5:]])
+    assert row_err(got, oracle(cfg, w, toks)[5:]) < TOL["float32"]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_other_sizes_odd_and_one(tmp_path, dt):
+    """Sizes that are no multiples of 8, one head, one expert group, top 1, no bigram table, rotation of only part of the rotated entries."""
+    from llm_quest_amd import registry
+
+    layers = [(U.latent(heads=1, dim=20, rot_dim=6, vdim=36, q_rank=28, kv_rank=44, rot_dims=4), U.moe(experts=5, top=1, groups=1, keep=1, ff=18)),
+              (U.gla(heads=1, dim=10, vdim=70, tau=1.0), U.moe(experts=4, top=4, groups=2, keep=2, ff=30)),
+              (U.latent(heads=7, dim=12, rot_dim=6, vdim=20, q_rank=36, kv_rank=44, kv_from=0, rot_dims=4), None),
+              (U.gla(heads=4, dim=36, vdim=12, tau=20.0), U.moe(experts=70, top=6, groups=7, keep=3, ff=10))]
+    cfg = U.make_config(layers, width=100, vocab=77, eps=1e-6, alpha=1.0, embed_scale=1.0, bigram=None)
+    w = U.make_weights(cfg, 5, decay_rank=5)
+    model = registry.load_model(U.save(str(tmp_path), cfg, w), dt, DEV)
+    toks = tokens(40, cfg["vocab"], 6)
+    want = G.forward(toks, w, cfg, torch.float32)
+    b = batch_of(model)
+    got = [b.step([("a", toks[:29])], [list(range(29))])] + [b.step([("a", [t])]) for t in toks[29:]]
+    assert model_err(torch.cat(got), want, dt) < TOL[dt]
+
+
+def test_greedy_generation_through_the_entry_point(models):
+    from llm_quest_amd.generate import generate_ragged
+
+    ms, cfg, w = models
+    prompts = [tokens(n, cfg["vocab"], 40 + n) for n in (4, 19, 9)]
+    out = generate_ragged(ms["float32"], prompts, max_gen=10)
+    for p, gen in zip(prompts, out):
+        assert len(gen) == 10
+        seq = list(p)
+        for t in gen:
+            lg = G.forward(seq, w, cfg, torch.float32)[-1]
+            top = torch.topk(lg, 2)
+            if int(top.indices[0]) != t:
+                assert float(top.values[0] - top.values[1]) < 1e-4, "greedy token differs from the oracle's without a near tie"
+                break
+            seq.append(t)
+    # eos ends a sequence early and the others go on
+    first = out[1][2]
+    out2 = generate_ragged(ms["float32"], prompts, max_gen=10, eos_ids=[first])
+    assert out2[1] == out[1][: out[1].index(first)] and out2[0][: len(out2[0])] == out[0][: len(out2[0])]
+
+
+# ------------------------------------------------------------------------------------------------------------------- mechanisms alone
+def test_embedding_first_token_and_large_hash():
+    from llm_quest_amd import kernels_seq as S
+
+    vocab, width, buckets, mp, mc = 60000, 24, 1009, 1000003, 999983  # prev * mul_prev overflows 32 bits
+    g = torch.Generator().manual_seed(0)
+    table, bigram = torch.randn(vocab, width, generator=g).to(BF16), torch.randn(buckets + 1, width, generator=g).to(BF16)
+    tok, prev = [59999, 0, 31337, 59998], [-1, 59999, 0, 59997]
+    got = S.embed_hash(dev_i32(tok), dev_i32(prev), table.to(DEV), 0.25, bigram.to(DEV), buckets, mp, mc).cpu()
+    for i, (t, p) in enumerate(zip(tok, prev)):
+        row = buckets if p < 0 else (p * mp + t * mc) % buckets
+        assert torch.equal(got[i], table[t].float() * 0.25 + bigram[row].float())
+
+
+def test_rotary_and_latent_rows_at_large_positions():
+    from llm_quest_amd import kernels_seq as S
+
+    T, H, n, dims, start, base = 9, 3, 22, 10, 8, 500000.0
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(T, H * n, generator=g)
+    pos = [0, 1, 2, 63, 64, 1000, 4095, 4096, 100000]
+    freq = S.rope_frequencies(dims, base, DEV)
+    dst = torch.zeros(T, H * n, device=DEV)
+    S.rope_heads(x.to(DEV), H, n, n, 0, dst, n, 0, start, dims, freq, dev_i32(pos))
+    xv = x.view(T, H, n).clone()
+    xv[..., start : start + dims] = G.rotate_pairs(xv[..., start : start + dims].double(), torch.tensor(pos), dims, base).float()
+    assert (dst.cpu().view(T, H, n)[:8] - xv[:8]).abs().max() < 2e-3  # angle p * f rounds to fp32: up to p * 2^-24 radians
+    assert (dst.cpu().view(T, H, n)[:5] - xv[:5]).abs().max() < 1e-5
+    assert (dst.cpu().view(T, H, n) - xv).abs().max() < 5e-2
+    rank, rot, rd = 20, 12, 8
+    src, wgt = torch.randn(T, rank + rot, generator=g), 1 + 0.1 * torch.randn(rank, generator=g)
+    cache = torch.zeros(40, rank + rot, device=DEV)
+    rows = [3, 39, 0, 7, 8, 21, 22, 23, 30]
+    S.latent_kv_append(src.to(DEV), rank, rot, wgt.to(DEV), 1e-5, dev_i32(pos), dev_i32(rows), S.rope_frequencies(rd, base, DEV), rd, cache)
+    want_c = G.rms_unit(src[:, :rank], 1e-5) * wgt
+    want_r = G.rotate_pairs(src[:, rank:].double(), torch.tensor(pos), rd, base).float()
+    got = cache.cpu()[rows]
+    assert (got[:, :rank] - want_c).abs().max() < 1e-5 and (got[:5, rank:] - want_r[:5]).abs().max() < 1e-5 and (got[:, rank:] - want_r).abs().max() < 5e-2
+    untouched = sorted(set(range(40)) - set(rows))
+    assert float(cache.cpu()[untouched].abs().sum()) == 0.0
+
+
+def _attention_reference(q, k1, k2, v, past, scale):
+    """q [n, H, D1+D2], k1 [L, H, D1], k2 [L, D2], v [L, H, DV]: row i sees keys j <= past + i."""
+    n, H, _ = q.shape
+    D1 = k1.shape[-1]
+    out = torch.zeros(n, H, v.shape[-1], dtype=torch.float64)
+    for i in range(n):
+        L = past + i + 1
+        s = (torch.einsum("hd,jhd->hj", q[i, :, :D1], k1[:L]) + q[i, :, D1:] @ k2[:L].T) * scale
+        out[i] = torch.einsum("hj,jhd->hd", torch.softmax(s, -1), v[:L])
+    return out
+
+
+@pytest.mark.parametrize("dt", [F32, BF16])
+@pytest.mark.parametrize("far", [0, 1, 63, 64, 65, 127, 128, 300, 383])
+def test_attention_finds_one_far_key_among_hundreds(dt, far):
+    """One key's score stands out (the last query is a multiple of that key): the output must be that key's value, wherever the key lies -- first rows,
+    the borders of the 64-key steps, the very last visible key -- in the per-head form (prompt) and in the shared-key form with a past (decoding)."""
+    from llm_quest_amd import kernels_seq as S
+
+    H, D1, D2, DV, L = 3, 24, 8, 40, 384
+    g = torch.Generator().manual_seed(far)
+    k1, k2, v = torch.randn(L, H, D1, generator=g), torch.randn(L, D2, generator=g), torch.randn(L, H, DV, generator=g)
+    k1, k2, v = (t.to(dt).float() for t in (k1, k2, v))  # the kernel sees exactly these values in both dtypes
+    q = torch.randn(L, H, D1 + D2, generator=g)
+    q[-1] = 3.0 * torch.cat([k1[far], k2[far].expand(H, D2)], -1)
+    scale = 0.3
+    # prompt form: per-head keys and values of this step, no past
+    want = _attention_reference(q.double(), k1.double(), k2.double(), v.double(), 0, scale)
+    out = torch.empty(L, H * DV, dtype=dt, device=DEV)
+    z = dev_i32([0])
+    S.latent_attn(q.view(L, -1).to(DEV), k1.view(L, -1).to(dt).to(DEV), k2.to(dt).to(DEV), v.view(L, -1).to(dt).to(DEV), out, H, 1, D1, D2, DV, D1 + D2, D1, DV, DV,
+                  (z, dev_i32([L]), z, z, z, z), L, scale)
+    tol = 1e-5 if dt == F32 else 2e-2
+    assert rel(out.view(L, H, DV), want) < tol
+    assert rel(out.view(L, H, DV)[-1], v[far]) < 0.05, "the far key's value did not come through"
+    # shared-key form: one key / value row set for all heads (the cache rows), the last 3 rows are new, the rest is the past; rows start at an offset
+    ks, vs = k1[:, 0], k1[:, 0]  # keys are also the values, as with cached latent rows
+    qs = torch.randn(3, H, D1 + D2, generator=g)
+    qs[-1] = 3.0 * torch.cat([ks[far], k2[far]], -1).expand(H, D1 + D2)
+    want = _attention_reference(qs.double(), ks[:, None].expand(L, H, D1).double(), k2.double(), vs[:, None].expand(L, H, D1).double(), L - 3, scale)
+    off = 5
+    rows = torch.zeros(off + L, D1 + D2)
+    rows[off:, :D1], rows[off:, D1:] = ks, k2
+    rows = rows.to(dt).to(DEV)
+    out = torch.empty(3, H * D1, dtype=dt, device=DEV)
+    o5 = dev_i32([off])
+    S.latent_attn(qs.view(3, -1).to(DEV), rows, rows[:, D1:], rows, out, H, 4, D1, D2, D1, D1 + D2, 0, 0, D1, (z, dev_i32([3]), dev_i32([L - 3]), o5, o5, o5), 3, scale)
+    assert rel(out.view(3, H, D1), want) < tol
+    assert rel(out.view(3, H, D1)[-1], ks[far].expand(H, D1)) < 0.05
+
+
+@pytest.mark.parametrize("dt", [F32, BF16])
+def test_gla_kernel_carries_state_over_cuts_and_keeps_a_far_token(dt):
+    from llm_quest_amd import kernels_seq as S
+
+    H, dk, dv, T, tau = 2, 20, 70, 150, 4.0
+    g = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(T, H * n, generator=g).to(dt) for n in (dk, dk, dv))
+    z = 6.0 + torch.randn(T, H * dk, generator=g)  # decays close to one: the first token stays visible to the end
+    k[0] *= 20.0
+    bias = 0.5 * torch.randn(H * dk, generator=g)
+    qf, kf, vf = q.float().view(T, H, dk), k.float().view(T, H, dk), v.float().view(T, H, dv)
+    a = torch.sigmoid((z + bias).double()).pow(1 / tau).view(T, H, dk)
+    S_ = torch.zeros(H, dk, dv, dtype=torch.float64)
+    want = torch.zeros(T, H, dv, dtype=torch.float64)
+    for t in range(T):
+        S_ = a[t].unsqueeze(-1) * S_ + kf[t].double().unsqueeze(-1) * vf[t].double().unsqueeze(-2)
+        want[t] = torch.einsum("hkv,hk->hv", S_, qf[t].double() * dk ** -0.5)
+    state = torch.zeros(3, H, dk, dv, device=DEV)
+    state[0] = state[2] = 99.0  # other slots: must stay as they are
+    got, at = [], 0
+    for n in [1, 7, 8, 9, 16, 1, 1, 2, 105]:  # cuts around the kernel's groups of 8 tokens
+        sl = slice(at, at + n)
+        got.append(S.gla(q[sl].to(DEV), k[sl].to(DEV), v[sl].to(DEV), z[sl].to(DEV), bias.to(DEV), 1 / tau, dk ** -0.5, dev_i32([0, n]), dev_i32([1]), state, H, dk, dv))
+        at += n
+    assert at == T
+    assert rel(torch.cat(got).view(T, H, dv), want) < 2e-5
+    assert rel(state[1], S_) < 2e-5 and float((state[0] - 99).abs().max()) == 0 and float((state[2] - 99).abs().max()) == 0
+    contribution = torch.einsum("hk,hv,hk->hv", (a[1:].prod(0) * kf[0].double()), vf[0].double(), qf[-1].double() * dk ** -0.5)
+    assert float(contribution.norm() / want[-1].norm()) > 0.5, "the test's far token does not dominate the last output"
+
+
+def test_router_matches_the_oracle_also_with_negative_choices_and_many_experts():
+    from llm_quest_amd import kernels_seq as S
+
+    for E, top, groups, keep, corr_mean in [(8, 2, 2, 1, 0.0), (12, 3, 4, 2, -2.0), (160, 6, 8, 3, -0.4), (70, 5, 70, 9, 0.1), (6, 6, 1, 1, 0.0), (200, 1, 4, 4, -3.0)]:
+        g = torch.Generator().manual_seed(E)
+        logits, corr = 2 * torch.randn(37, E, generator=g), corr_mean + 0.3 * torch.randn(E, generator=g)
+        r = {"experts": E, "top": top, "groups": {"count": groups, "keep": keep}, "scale": 1.7}
+        w = {"x.router": torch.eye(E), "x.correction": corr}
+        ids, wt = G.route(logits, w, "x.", r)
+        gi, gw = S.moe_route(logits.to(DEV), corr.to(DEV), top, groups, keep, 1.7)
+        assert torch.equal(gi.cpu().long(), ids), (E, top, groups, keep)
+        assert torch.allclose(gw.cpu(), wt, atol=1e-6)
+        offs, perm = S.moe_dispatch(gi.view(-1), E)
+        offs, perm = offs.cpu().tolist(), perm.cpu().tolist()
+        flat = ids.view(-1).tolist()
+        assert offs[0] == 0 and offs[-1] == len(flat) and sorted(perm) == list(range(len(flat)))
+        for e in range(E):
+            assert all(flat[i] == e for i in perm[offs[e] : offs[e + 1]]) and perm[offs[e] : offs[e + 1]] == sorted(perm[offs[e] : offs[e + 1]])
+
+
+@pytest.mark.parametrize("dt", [F32, BF16])
+def test_strided_and_grouped_products(dt):
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(4)
+    # per-head product with the weight read [in, out] (n fastest) and [out, in]
+    T, H, dn, R, extra = 37, 3, 20, 44, 6
+    a = torch.randn(T, H * (dn + extra), generator=g).to(dt)
+    wk = torch.randn(H * dn, R, generator=g).to(BF16)
+    c = torch.zeros(T, H * (R + 2), device=DEV)
+    S.bgemm(a.to(DEV), wk.to(DEV), c, T, R, dn, batch=H, lda=a.shape[1], a_bs=dn + extra, sbn=1, sbk=R, b_bs=dn * R, ldc=H * (R + 2), c_bs=R + 2)
+    want = torch.einsum("thd,hdr->thr", a.float().view(T, H, dn + extra)[..., :dn], wk.float().view(H, dn, R))
+    assert rel(c.view(T, H, R + 2)[..., :R], want) < 1e-5
+    wv = torch.randn(H * 28, R, generator=g).to(BF16)
+    a2 = torch.randn(T, H * R, generator=g).to(dt)
+    c2 = torch.empty(T, H * 28, dtype=dt, device=DEV)
+    S.bgemm(a2.to(DEV), wv.to(DEV), c2, T, 28, R, batch=H, lda=H * R, a_bs=R, sbn=R, sbk=1, b_bs=28 * R, ldc=H * 28, c_bs=28)
+    assert rel(c2.view(T, H, 28), torch.einsum("thr,hvr->thv", a2.float().view(T, H, R), wv.float().view(H, 28, R))) < (1e-5 if dt == F32 else 4e-3)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_mixture_of_experts_alone(dt):
+    from llm_quest_amd.common.mixers import GroupedSigmoidMoE
+
+    cfg = U.make_config([(U.gla(), U.moe(experts=10, top=3, groups=5, keep=2, ff=36))], width=88)
+    w = U.make_weights(cfg, 8)
+    m = GroupedSigmoidMoE(88, 36, 10, 3, 5, 2, 2.5)
+    m.w_router.data.copy_(w["l0.mlp.router"])
+    m.correction.data.copy_(w["l0.mlp.correction"])
+    m.w_up.data.copy_(torch.stack([w[f"l0.mlp.e{e}.up"] for e in range(10)]))
+    m.w_down.data.copy_(torch.stack([w[f"l0.mlp.e{e}.down"] for e in range(10)]))
+    m = m.to(DEV)
+    x = torch.randn(150, 88, generator=torch.Generator().manual_seed(9))
+    act = F32 if dt == "float32" else BF16
+    h = x.to(act)
+    got = m.step(x.to(DEV), h.to(DEV)).view(150, 3, 88).sum(1)
+    wf = {k: v.float() for k, v in w.items()}
+    ids_x, _ = G.route(x, wf, "l0.mlp.", cfg["layers"][0]["mlp"]["router"])
+    want = torch.zeros(150, 88)
+    _, wt = G.route(x, wf, "l0.mlp.", cfg["layers"][0]["mlp"]["router"])
+    for t in range(150):
+        for j in range(3):
+            e = int(ids_x[t, j])
+            want[t] += wt[t, j] * (wf[f"l0.mlp.e{e}.down"] @ (torch.relu(wf[f"l0.mlp.e{e}.up"] @ h[t].float()) ** 2))
+    assert rel(got, want) < (1e-5 if dt == "float32" else 1e-2)
+
+
+def test_post_sum_layernorm_and_head_norm():
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(6)
+    for width in (72, 100, 256, 1000):
+        x, y = 3 + torch.randn(13, width, generator=g), torch.randn(13 * 2, width, generator=g)
+        w, b = torch.randn(width, generator=g), torch.randn(width, generator=g)
+        out, cast = S.add_layernorm(x.to(DEV), w.to(DEV), b.to(DEV), 1e-5, 3.0, y.to(DEV), 2, BF16)
+        want = G.layer_norm((3.0 * x + y.view(13, 2, width).sum(1)).double(), w.double(), b.double(), 1e-5)
+        assert (out.cpu() - want).abs().max() < 2e-5 and torch.equal(cast.cpu(), out.cpu().to(BF16))
+    o, gate, wn = torch.randn(11, 3 * 70, generator=g), torch.randn(11, 3 * 70, generator=g), torch.randn(70, generator=g)
+    got = S.gated_headnorm(o.to(DEV), wn.to(DEV), gate.to(DEV), 3, 70, 1e-5, F32)
+    want = (G.rms_unit(o.view(11, 3, 70).double(), 1e-5) * wn.double()).view(11, -1) * torch.nn.functional.silu(gate.double())
+    assert (got.cpu() - want).abs().max() < 1e-5
