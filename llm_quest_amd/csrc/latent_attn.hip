@@ -164,6 +164,184 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
     }
 }
 
+
+// ---- MFMA path (bf16 keys / values).  A workgroup is four waves; wave w owns query rows 32 w .. 32 w + 31 of a 128-row tile and keeps their Q fragments
+// (bf16) in registers.  Scores are computed transposed, S^T = K Q^T (v_mfma_f32_32x32x8_bf16_1k: A = 32 keys x 8 features from LDS, B = the lane's own
+// query), so a lane holds 16 of every 32 keys of ONE query: the softmax statistics are lane-local plus one exchange with lane ^ 32, the rescale factor
+// of the transposed output O^T = V^T P^T is lane-local too, and P (bf16) is the B operand of that product as it stands in registers.  The key tile lies in
+// LDS as [64 keys][DKP] (main part and rotated part side by side, zero padded), the value tile transposed as [DVP][64 keys].
+#define MQ 128
+#define MKT 64
+template <int DKS, int NVB>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, int vec_ok) {
+    constexpr int DKP = DKS * 8, DVP = NVB * 32, KLD = DKP + 4, VLD = MKT + 4;
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[MKT * KLD];
+    __shared__ __attribute__((aligned(16))) bf16_t Vt[DVP * VLD];
+    const int s = blockIdx.z, tm = MQ / p.hm;
+    const int tok0 = blockIdx.x * tm, head0 = blockIdx.y * p.hm;
+    const int n_new = p.n_new[s], past = p.past[s];
+    if (tok0 >= n_new) return;
+    const int64_t qr0 = p.q_row0[s], k1r0 = p.k1_row0[s], k2r0 = p.k2_row0[s], vr0 = p.v_row0[s];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, ln = lane & 31, hf = lane >> 5;
+    const int DK = p.D1 + p.D2;
+    const bf16_t* K1 = (const bf16_t*)p.K1;
+    const bf16_t* K2 = (const bf16_t*)p.K2;
+    const bf16_t* V = (const bf16_t*)p.V;
+    // this lane's query
+    const int row = 32 * wave + ln, tok = tok0 + row / p.hm, head = head0 + row % p.hm;
+    const bool row_ok = tok < n_new && head < p.H;
+    const int lim = row_ok ? past + tok : -1;
+    bf16x4 qf[DKS];
+    {
+        const float* qrow = p.Q + (qr0 + (row_ok ? tok : 0)) * p.ldq + (int64_t)(row_ok ? head : 0) * p.q_hs;
+#pragma unroll
+        for (int st = 0; st < DKS; ++st) {
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int d = 8 * st + 4 * hf + j;
+                v[j] = (row_ok && d < DK) ? qrow[d] : 0.f;
+            }
+            const unsigned lo = pack_bf2(v[0], v[1]), hi = pack_bf2(v[2], v[3]);
+            u32x2 pk = {lo, hi};
+            qf[st] = __builtin_bit_cast(bf16x4, pk);
+        }
+    }
+    const int n_keys = past + min(tok0 + tm, n_new);
+    // the last key any row of this WAVE may see (its rows are consecutive, so its last valid row has the largest limit)
+    int wave_lim = lim;
+#pragma unroll
+    for (int of = 32; of > 0; of >>= 1) wave_lim = max(wave_lim, __shfl_xor(wave_lim, of, 64));
+    f32x16 oacc[NVB];
+#pragma unroll
+    for (int vb = 0; vb < NVB; ++vb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[vb][i] = 0.f;
+    const float NEG = -__builtin_huge_valf();
+    float m_run = NEG, l_run = 0.f;
+    const float sc2 = p.scale * 1.4426950408889634f;
+
+    for (int j0 = 0; j0 < n_keys; j0 += MKT) {
+        __syncthreads();
+        // ---- key tile -> LDS
+        for (int c = tid; c < MKT * DKS; c += 256) {
+            const int key = c / DKS, d0 = (c % DKS) * 8, j = j0 + key;
+            u32x4 val = {0u, 0u, 0u, 0u};
+            if (j < n_keys) {
+                if (vec_ok && d0 + 8 <= p.D1) {
+                    val = *(const u32x4*)(K1 + (k1r0 + j) * p.ldk1 + (int64_t)head0 * p.k1_hs + d0);
+                } else if (vec_ok && d0 >= p.D1 && d0 + 8 <= DK) {
+                    val = *(const u32x4*)(K2 + (k2r0 + j) * p.ldk2 + (d0 - p.D1));
+                } else {
+                    bf16_t e[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const int d = d0 + i;
+                        e[i] = d < p.D1 ? K1[(k1r0 + j) * p.ldk1 + (int64_t)head0 * p.k1_hs + d] : (d < DK ? K2[(k2r0 + j) * p.ldk2 + (d - p.D1)] : (bf16_t)0);
+                    }
+                    val = u32x4{(unsigned)e[0] | ((unsigned)e[1] << 16), (unsigned)e[2] | ((unsigned)e[3] << 16), (unsigned)e[4] | ((unsigned)e[5] << 16),
+                                (unsigned)e[6] | ((unsigned)e[7] << 16)};
+                }
+            }
+            u32x2* dst = (u32x2*)&Ks[key * KLD + d0];  // rows are 8-byte aligned (KLD % 4 == 0)
+            dst[0] = u32x2{val[0], val[1]};
+            dst[1] = u32x2{val[2], val[3]};
+        }
+        // ---- value tile -> LDS, transposed
+        for (int c = tid; c < MKT * (DVP / 8); c += 256) {
+            const int key = c % MKT, v0 = (c / MKT) * 8, j = j0 + key;
+            bf16_t e[8];
+            if (j < n_keys && vec_ok && v0 + 8 <= p.DV) {
+                const u32x4 val = *(const u32x4*)(V + (vr0 + j) * p.ldv + (int64_t)head0 * p.v_hs + v0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) e[2 * i] = (bf16_t)(val[i] & 0xffffu), e[2 * i + 1] = (bf16_t)(val[i] >> 16);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) e[i] = (j < n_keys && v0 + i < p.DV) ? V[(vr0 + j) * p.ldv + (int64_t)head0 * p.v_hs + v0 + i] : (bf16_t)0;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) Vt[(v0 + i) * VLD + key] = e[i];
+        }
+        __syncthreads();
+        if (j0 > wave_lim) continue;  // every key of this step lies behind the wave's rows (the barriers above are still reached by all)
+        // ---- S^T = K Q^T: two blocks of 32 keys
+        f32x16 sacc[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
+#pragma unroll
+            for (int st = 0; st < DKS; ++st) {
+                const bf16x4 a = *(const bf16x4*)&Ks[(kb * 32 + ln) * KLD + 8 * st + 4 * hf];
+                sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a, qf[st], sacc[kb], 0, 0, 0);
+            }
+        }
+        // ---- online softmax for the lane's query (keys kb * 32 + 8 g + 4 hf + i)
+        float mx = NEG;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int j = j0 + kb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
+                const float v = j <= lim ? sacc[kb][r] * sc2 : NEG;
+                sacc[kb][r] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float base = m_new == NEG ? 0.f : m_new;
+        const float f = exp2f(m_run - base);
+        float sum = 0.f;
+        bf16x4 pf[8];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float e[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    e[i] = exp2f(sacc[kb][4 * g + i] - base);
+                    sum += e[i];
+                }
+                u32x2 pk = {pack_bf2(e[0], e[1]), pack_bf2(e[2], e[3])};
+                pf[kb * 4 + g] = __builtin_bit_cast(bf16x4, pk);
+            }
+        sum += __shfl_xor(sum, 32, 64);
+        l_run = l_run * f + sum;
+        m_run = m_new;
+        // ---- O^T <- O^T * f + V^T P^T
+#pragma unroll
+        for (int vb = 0; vb < NVB; ++vb) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[vb][i] *= f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                const bf16x4 a = *(const bf16x4*)&Vt[(vb * 32 + ln) * VLD + 8 * ks + 4 * hf];
+                oacc[vb] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a, pf[ks], oacc[vb], 0, 0, 0);
+            }
+        }
+    }
+    if (!row_ok) return;
+    const float inv = 1.0f / l_run;
+    bf16_t* orow = (bf16_t*)p.O + (qr0 + tok) * p.ldo + (int64_t)head * p.o_hs;
+#pragma unroll
+    for (int vb = 0; vb < NVB; ++vb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int dv = vb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
+            if (dv < p.DV) orow[dv] = f2bf(oacc[vb][r] * inv);
+        }
+}
+
+template <int DKS>
+static int launch_mfma(const LatAttnArgs& p, dim3 grid, int vec_ok, hipStream_t st) {
+    if (p.DV <= 32) latent_attn_mfma_kernel<DKS, 1><<<grid, 256, 0, st>>>(p, vec_ok);
+    else if (p.DV <= 64) latent_attn_mfma_kernel<DKS, 2><<<grid, 256, 0, st>>>(p, vec_ok);
+    else if (p.DV <= 128) latent_attn_mfma_kernel<DKS, 4><<<grid, 256, 0, st>>>(p, vec_ok);
+    else latent_attn_mfma_kernel<DKS, 8><<<grid, 256, 0, st>>>(p, vec_ok);
+    return 0;
+}
+
 extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, int D2, int DV, const float* Q, int64_t ldq, int q_hs, const void* K1, int64_t ldk1,
                                  int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
                                  const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
@@ -171,7 +349,8 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
     MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && max_new > 0 && H > 0 && D1 > 0 && D2 >= 0 && DV > 0 && DV <= 512 && Q && K1 && V && O && (D2 == 0 || K2),
                   "latent_attn: bad arguments (value width <= 512)");
     MI355_REQUIRE(dt == MI355_DT_BF16 || dt == MI355_DT_F32, "latent_attn: bad dtype");
-    MI355_REQUIRE(hm >= 1 && hm <= AM && AM % hm == 0 && (hm == 1 || (k1_hs == 0 && v_hs == 0)), "latent_attn: several heads per tile need shared keys and values (head stride 0)");
+    MI355_REQUIRE(hm >= 1 && hm <= AM && AM % hm == 0 && (hm == 1 || (k1_hs == 0 && v_hs == 0)), "latent_attn: several heads per tile (a power of two <= 32) need shared keys and values (head stride 0)");
+    MI355_REQUIRE(!use_mfma || dt == MI355_DT_BF16, "latent_attn: the MFMA path takes bf16 keys and values");
     MI355_REQUIRE(q_row0 && n_new && past && k1_row0 && k2_row0 && v_row0, "latent_attn: sequence descriptors missing");
     MI355_REQUIRE(ldq >= (int64_t)(H - 1) * q_hs + D1 + D2 && ldo >= (int64_t)(H - 1) * o_hs + DV && ldk1 >= (int64_t)(H - 1) * k1_hs + D1 && ldv >= (int64_t)(H - 1) * v_hs + DV &&
                       (D2 == 0 || ldk2 >= D2),
@@ -183,11 +362,22 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
     p.D1 = D1, p.D2 = D2, p.DV = DV, p.H = H, p.hm = hm, p.dt = dt;
     p.q_row0 = q_row0, p.n_new = n_new, p.past = past, p.k1_row0 = k1_row0, p.k2_row0 = k2_row0, p.v_row0 = v_row0;
     p.scale = scale;
-    const int tm = AM / hm;
+    const bool mfma = use_mfma && D1 + D2 <= 320 && DV <= 256;  // what the MFMA kernel keeps in registers; larger heads take the FMA path
+    const int tm = (mfma ? MQ : AM) / hm;
     const int64_t gx = ((int64_t)max_new + tm - 1) / tm, gy = (H + hm - 1) / hm;
     MI355_REQUIRE(gy <= 65535 && gx < ((int64_t)1 << 31), "latent_attn: grid too large");
     const dim3 grid((unsigned)gx, (unsigned)gy, n_seq);
-    (void)use_mfma;
+    if (mfma) {
+        const int vec_ok = D1 % 8 == 0 && D2 % 8 == 0 && DV % 8 == 0 && ldk1 % 8 == 0 && ldk2 % 8 == 0 && ldv % 8 == 0 && k1_hs % 8 == 0 && v_hs % 8 == 0 &&
+                           ((uintptr_t)K1 & 15) == 0 && ((uintptr_t)K2 & 15) == 0 && ((uintptr_t)V & 15) == 0;
+        const int DK = D1 + D2;
+        if (DK <= 64) launch_mfma<8>(p, grid, vec_ok, ST(stream));
+        else if (DK <= 128) launch_mfma<16>(p, grid, vec_ok, ST(stream));
+        else if (DK <= 192) launch_mfma<24>(p, grid, vec_ok, ST(stream));
+        else launch_mfma<40>(p, grid, vec_ok, ST(stream));
+        MI355_LAUNCH_CHECK("latent_attn(mfma)");
+        return 0;
+    }
     if (DV <= 64) latent_attn_fma_kernel<1><<<grid, 256, 0, ST(stream)>>>(p);
     else if (DV <= 128) latent_attn_fma_kernel<2><<<grid, 256, 0, ST(stream)>>>(p);
     else if (DV <= 256) latent_attn_fma_kernel<4><<<grid, 256, 0, ST(stream)>>>(p);
