@@ -535,6 +535,8 @@ int mi355_gated_headnorm(int64_t tokens, int H, int D, const float* o, const flo
  * o fp32 [tokens, H * dv].  dk <= 256. */
 int mi355_gla_fwd(int n_seq, const int* seq_off, const int* slot, int H, int dk, int dv, const void* q, const void* k, const void* v, const void* z, int dt,
                   int z_dt, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldz, const float* zbias, float inv_tau, float qscale, float* state, float* o, void* stream);
+/* logits[t, e] = sum_k x[t, k] W[e, k]: fp32 rows (pitch ldx) against a bf16 matrix [E, K] (pitch ldw), fp32 FMA; out fp32 [tokens, E]. */
+int mi355_router_logits(int64_t tokens, int E, int K, const float* x, int64_t ldx, const void* W, int64_t ldw, float* out, void* stream);
 /* Grouped sigmoid router: s = sigmoid(logits), choice = s + correction (may be NULL); a group (E / groups neighbours) scores the sum of its two
  * largest choices, experts outside the `keep` best groups are excluded, the `top` largest choices win; wts = s / (sum + 1e-20) * scale.
  * ids int32 [tokens, top] in descending order of choice, wts fp32 [tokens, top]. */
@@ -551,11 +553,13 @@ int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t
                 const float* row_scale, int epi, int use_mfma, void* stream);
 /* Causal attention with two-part keys over ragged batches: sequence s has n_new[s] query rows starting at row q_row0[s], `past[s]` earlier keys;
  * key j of it is K1 row k1_row0[s] + j (head stride k1_hs, D1 wide), K2 row k2_row0[s] + j (shared by heads, D2 wide), value row v_row0[s] + j.
- * Q fp32 [.., H, D1 + D2]; K1 / K2 / V / O of dtype dt.  A tile covers 32 / hm tokens x hm heads (hm > 1 needs k1_hs == v_hs == 0). */
+ * Q fp32 [.., H, D1 + D2]; K1 / K2 / V / O of dtype dt.  A tile covers 32 / hm tokens x hm heads (hm > 1 needs k1_hs == v_hs == 0); the MFMA path (bf16,
+ * D1 + D2 <= 320, DV <= 256) 128 / hm tokens, and with splits > 1 deals a tile's keys to that many workgroups whose partial results meet in ws
+ * (n_seq * head tiles * token tiles * splits * 128 * (2 + DV rounded up to 32 / 64 / 128 / 256) floats). */
 int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, int D2, int DV, const float* Q, int64_t ldq, int q_hs, const void* K1, int64_t ldk1,
                       int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
                       const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
-                      int use_mfma, void* stream);
+                      int use_mfma, int splits, float* ws, int64_t ws_floats, void* stream);
 
 #ifdef __cplusplus
 }

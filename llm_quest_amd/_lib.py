@@ -108,10 +108,11 @@ SIGNATURES = {
     "mi355_rope_heads": [_L, _I, _I, _P, _I, _L, _I, _I, _P, _L, _I, _I, _I, _I, _P, _P, _P],
     "mi355_gated_headnorm": [_L, _I, _I, _P, _P, _P, _I, _L, _F, _P, _I, _L, _P],
     "mi355_gla_fwd": [_I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _I, _L, _L, _L, _L, _P, _F, _F, _P, _P, _P],
+    "mi355_router_logits": [_L, _I, _I, _P, _L, _P, _L, _P, _P],
     "mi355_moe_route": [_L, _I, _I, _I, _I, _P, _P, _F, _P, _P, _P],
     "mi355_moe_dispatch": [_L, _I, _P, _P, _P, _P],
     "mi355_bgemm": [_I, _I, _I, _I, _P, _I, _L, _L, _P, _I, _L, _L, _L, _P, _I, _L, _L, _P, _P, _I, _P, _P, _I, _I, _P],
-    "mi355_latent_attn": [_I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _F, _I, _P],
+    "mi355_latent_attn": [_I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _F, _I, _I, _P, _L, _P],
     # measurement aid (csrc/probe.hip)
     "mi355_mfma_pipe_probe": [_I, _I, _P, _P],
     # stand-alone RoPE and dropout (csrc/rope_dropout.hip, csrc/attention_generic.hip)

@@ -40,6 +40,7 @@ class SeqStep:
         cache.reserve(max(p + n for p, n in zip(past, n_new)))
         cap = cache.capacity
         self.T, self.n_seq, self.max_new = len(tok), len(slots), max(n_new)
+        self.max_keys = max(p + n for p, n in zip(past, n_new))
         self.fresh = all(p == 0 for p in past)
         self.host_seq_off = seq_off
         row0 = [s * cap for s in slots]
@@ -136,7 +137,7 @@ class LatentAttention(_Frozen):
                 hm *= 2
             ol = torch.empty((T, H * R), dtype=st.act_dtype, device=h.device)
             S.latent_attn(qf, cache2d, cache2d[:, R:], cache2d, ol, H, hm, R, dr, R, R + dr, 0, 0, R,
-                          (st.q_row0, st.n_new, st.past, st.cache_row0, st.cache_row0, st.cache_row0), st.max_new, self.scale)
+                          (st.q_row0, st.n_new, st.past, st.cache_row0, st.cache_row0, st.cache_row0), st.max_new, self.scale, max_keys=st.max_keys)
             ctx = torch.empty((T, H * dv), dtype=st.act_dtype, device=h.device)
             S.bgemm(ol, self.w_ukv[H * dn :], ctx, T, dv, R, batch=H, lda=H * R, a_bs=R, sbn=R, sbk=1, b_bs=dv * R, ldc=H * dv, c_bs=dv)
         return S.linear(ctx, self.w_o)
@@ -202,8 +203,7 @@ class GroupedSigmoidMoE(_Frozen):
         """x32: the fp32 residual rows (the router reads them), h: the same rows in the activation dtype -> fp32 [T * top, width]."""
         self.prepare(h.device)
         T, E, top = h.shape[0], self.experts, self.top
-        logits = torch.empty((T, E), dtype=F32, device=h.device)
-        S.bgemm(x32, self.w_router, logits, T, E, self.width, mfma=False)
+        logits = S.router_logits(x32, self.w_router)
         ids, wts = S.moe_route(logits, self.correction32, top, self.groups, self.keep, self.scale)
         offs, perm = S.moe_dispatch(ids.view(-1), E)
         act = torch.empty((T * top, self.ff), dtype=h.dtype, device=h.device)

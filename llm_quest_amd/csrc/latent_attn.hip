@@ -24,6 +24,8 @@ struct LatAttnArgs {
     int D1, D2, DV, H, hm, dt;
     const int *q_row0, *n_new, *past, *k1_row0, *k2_row0, *v_row0;
     float scale;
+    int splits;  // MFMA path: a tile's keys are dealt to `splits` workgroups; partial (max, sum, output) rows go to ws and latent_attn_combine_kernel joins them
+    float* ws;   // per (sequence, head tile, token tile, split): 128 maxima | 128 sums | 128 x DVP unnormalised outputs
 };
 
 __device__ __forceinline__ float lda_dt(const void* p, int dt, int64_t i) { return dt == MI355_DT_F32 ? ((const float*)p)[i] : bf2f(((const bf16_t*)p)[i]); }
@@ -178,7 +180,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
     __shared__ __attribute__((aligned(16))) bf16_t Ks[MKT * KLD];
     __shared__ __attribute__((aligned(16))) bf16_t Vt[DVP * VLD];
     const int s = blockIdx.z, tm = MQ / p.hm;
-    const int tok0 = blockIdx.x * tm, head0 = blockIdx.y * p.hm;
+    const int tile = blockIdx.x / p.splits, split = blockIdx.x % p.splits;
+    const int tok0 = tile * tm, head0 = blockIdx.y * p.hm;
     const int n_new = p.n_new[s], past = p.past[s];
     if (tok0 >= n_new) return;
     const int64_t qr0 = p.q_row0[s], k1r0 = p.k1_row0[s], k2r0 = p.k2_row0[s], vr0 = p.v_row0[s];
@@ -207,7 +210,13 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
             qf[st] = __builtin_bit_cast(bf16x4, pk);
         }
     }
-    const int n_keys = past + min(tok0 + tm, n_new);
+    int n_keys = past + min(tok0 + tm, n_new);
+    int key_lo = 0;
+    if (p.splits > 1) {  // this workgroup's share: whole 64-key steps
+        const int span = ((n_keys + MKT - 1) / MKT + p.splits - 1) / p.splits * MKT;
+        key_lo = split * span;
+        n_keys = min(n_keys, key_lo + span);
+    }
     // the last key any row of this WAVE may see (its rows are consecutive, so its last valid row has the largest limit)
     int wave_lim = lim;
 #pragma unroll
@@ -221,7 +230,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
     float m_run = NEG, l_run = 0.f;
     const float sc2 = p.scale * 1.4426950408889634f;
 
-    for (int j0 = 0; j0 < n_keys; j0 += MKT) {
+    for (int j0 = key_lo; j0 < n_keys; j0 += MKT) {
         __syncthreads();
         // ---- key tile -> LDS
         for (int c = tid; c < MKT * DKS; c += 256) {
@@ -283,7 +292,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int j = j0 + kb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
-                const float v = j <= lim ? sacc[kb][r] * sc2 : NEG;
+                const float v = (j <= lim && j < n_keys) ? sacc[kb][r] * sc2 : NEG;
                 sacc[kb][r] = v;
                 mx = fmaxf(mx, v);
             }
@@ -321,6 +330,16 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
             }
         }
     }
+    if (p.splits > 1) {  // partial results; rows that see nothing keep max = -inf and sum = 0
+        const int64_t blk = (((int64_t)s * gridDim.y + blockIdx.y) * (gridDim.x / p.splits) + tile) * p.splits + split;
+        float* base = p.ws + blk * (int64_t)(MQ * (2 + DVP));
+        if (hf == 0) base[row] = m_run, base[MQ + row] = l_run;
+#pragma unroll
+        for (int vb = 0; vb < NVB; ++vb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) base[2 * MQ + (int64_t)row * DVP + vb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3)] = oacc[vb][r];
+        return;
+    }
     if (!row_ok) return;
     const float inv = 1.0f / l_run;
     bf16_t* orow = (bf16_t*)p.O + (qr0 + tok) * p.ldo + (int64_t)head * p.o_hs;
@@ -331,6 +350,38 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
             const int dv = vb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
             if (dv < p.DV) orow[dv] = f2bf(oacc[vb][r] * inv);
         }
+}
+
+// Joins the partial results of a tile's key splits: one wave per query row.
+__global__ __launch_bounds__(256) void latent_attn_combine_kernel(LatAttnArgs p, int DVP, int tiles, int gy, int n_seq) {
+    const int lane = threadIdx.x & 63;
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // (sequence, head tile, token tile, row)
+    const int row = (int)(item % MQ);
+    int64_t rest = item / MQ;
+    const int tile = (int)(rest % tiles);
+    rest /= tiles;
+    const int by = (int)(rest % gy), s = (int)(rest / gy);
+    if (s >= n_seq) return;
+    const int tm = MQ / p.hm, tok = tile * tm + row / p.hm, head = by * p.hm + row % p.hm;
+    if (tok >= p.n_new[s] || head >= p.H) return;
+    const int64_t blk0 = (((int64_t)s * gy + by) * tiles + tile) * p.splits;
+    const int64_t stride = (int64_t)MQ * (2 + DVP);
+    float m = -__builtin_huge_valf();
+    for (int i = 0; i < p.splits; ++i) m = fmaxf(m, p.ws[(blk0 + i) * stride + row]);
+    float l = 0.f;
+    for (int i = 0; i < p.splits; ++i) {
+        const float mi = p.ws[(blk0 + i) * stride + row];
+        if (mi != -__builtin_huge_valf()) l += p.ws[(blk0 + i) * stride + MQ + row] * exp2f(mi - m);
+    }
+    bf16_t* orow = (bf16_t*)p.O + ((int64_t)p.q_row0[s] + tok) * p.ldo + (int64_t)head * p.o_hs;
+    for (int dv = lane; dv < p.DV; dv += 64) {
+        float acc = 0.f;
+        for (int i = 0; i < p.splits; ++i) {
+            const float mi = p.ws[(blk0 + i) * stride + row];
+            if (mi != -__builtin_huge_valf()) acc += p.ws[(blk0 + i) * stride + 2 * MQ + (int64_t)row * DVP + dv] * exp2f(mi - m);
+        }
+        orow[dv] = f2bf(acc / l);
+    }
 }
 
 template <int DKS>
@@ -345,7 +396,7 @@ static int launch_mfma(const LatAttnArgs& p, dim3 grid, int vec_ok, hipStream_t 
 extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, int D2, int DV, const float* Q, int64_t ldq, int q_hs, const void* K1, int64_t ldk1,
                                  int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
                                  const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
-                                 int use_mfma, void* stream) {
+                                 int use_mfma, int splits, float* ws, int64_t ws_floats, void* stream) {
     MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && max_new > 0 && H > 0 && D1 > 0 && D2 >= 0 && DV > 0 && DV <= 512 && Q && K1 && V && O && (D2 == 0 || K2),
                   "latent_attn: bad arguments (value width <= 512)");
     MI355_REQUIRE(dt == MI355_DT_BF16 || dt == MI355_DT_F32, "latent_attn: bad dtype");
@@ -362,11 +413,19 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
     p.D1 = D1, p.D2 = D2, p.DV = DV, p.H = H, p.hm = hm, p.dt = dt;
     p.q_row0 = q_row0, p.n_new = n_new, p.past = past, p.k1_row0 = k1_row0, p.k2_row0 = k2_row0, p.v_row0 = v_row0;
     p.scale = scale;
+    p.splits = 1, p.ws = nullptr;
     const bool mfma = use_mfma && D1 + D2 <= 320 && DV <= 256;  // what the MFMA kernel keeps in registers; larger heads take the FMA path
     const int tm = (mfma ? MQ : AM) / hm;
     const int64_t gx = ((int64_t)max_new + tm - 1) / tm, gy = (H + hm - 1) / hm;
     MI355_REQUIRE(gy <= 65535 && gx < ((int64_t)1 << 31), "latent_attn: grid too large");
-    const dim3 grid((unsigned)gx, (unsigned)gy, n_seq);
+    dim3 grid((unsigned)gx, (unsigned)gy, n_seq);
+    if (mfma && splits > 1) {
+        const int DVPh = DV <= 32 ? 32 : DV <= 64 ? 64 : DV <= 128 ? 128 : 256;
+        const int64_t need = (int64_t)n_seq * gy * gx * splits * MQ * (2 + DVPh);
+        MI355_REQUIRE(splits <= 64 && ws && ws_floats >= need && gx * splits < ((int64_t)1 << 31), "latent_attn: key splits need a workspace of %lld floats", (long long)need);
+        p.splits = splits, p.ws = ws;
+        grid.x = (unsigned)(gx * splits);
+    }
     if (mfma) {
         const int vec_ok = D1 % 8 == 0 && D2 % 8 == 0 && DV % 8 == 0 && ldk1 % 8 == 0 && ldk2 % 8 == 0 && ldv % 8 == 0 && k1_hs % 8 == 0 && v_hs % 8 == 0 &&
                            ((uintptr_t)K1 & 15) == 0 && ((uintptr_t)K2 & 15) == 0 && ((uintptr_t)V & 15) == 0;
@@ -376,6 +435,12 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
         else if (DK <= 192) launch_mfma<24>(p, grid, vec_ok, ST(stream));
         else launch_mfma<40>(p, grid, vec_ok, ST(stream));
         MI355_LAUNCH_CHECK("latent_attn(mfma)");
+        if (p.splits > 1) {
+            const int DVPh = DV <= 32 ? 32 : DV <= 64 ? 64 : DV <= 128 ? 128 : 256;
+            const int64_t items = (int64_t)n_seq * gy * gx * MQ;
+            latent_attn_combine_kernel<<<(unsigned)((items + 3) / 4), 256, 0, ST(stream)>>>(p, DVPh, (int)gx, (int)gy, n_seq);
+            MI355_LAUNCH_CHECK("latent_attn(combine)");
+        }
         return 0;
     }
     if (DV <= 64) latent_attn_fma_kernel<1><<<grid, 256, 0, ST(stream)>>>(p);

@@ -114,11 +114,88 @@ __global__ __launch_bounds__(256) void add_layernorm_kernel(int64_t T, int width
     }
 }
 
+// The same for wide rows: one workgroup per row, 16-byte accesses (width % 4 == 0), thread t owns elements 4 (t + 256 j) .. + 4.
+template <int V4>
+__global__ __launch_bounds__(256) void add_layernorm_wide_kernel(int64_t T, int width, const float* __restrict__ x, float alpha, const void* __restrict__ y, int y_dt,
+                                                                 int64_t ldy, int parts, const float* __restrict__ w, const float* __restrict__ b, float eps,
+                                                                 float* __restrict__ out, void* __restrict__ cast, int cast_dt) {
+    __shared__ float red[2][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int64_t t = blockIdx.x; t < T; t += gridDim.x) {
+        f32x4 v[V4];
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < V4; ++j) {
+            const int i = 4 * (tid + 256 * j);
+            f32x4 a = {0.f, 0.f, 0.f, 0.f};
+            if (i < width) {
+                a = *(const f32x4*)(x + t * width + i) * alpha;
+                if (y) {
+                    f32x4 ys = {0.f, 0.f, 0.f, 0.f};
+                    for (int pp = 0; pp < parts; ++pp) {
+                        const int64_t o = (t * parts + pp) * ldy + i;
+                        if (y_dt == MI355_DT_F32) ys += *(const f32x4*)((const float*)y + o);
+                        else {
+                            const u32x2 r = *(const u32x2*)((const bf16_t*)y + o);
+                            ys += f32x4{__uint_as_float(r[0] << 16), __uint_as_float(r[0] & 0xffff0000u), __uint_as_float(r[1] << 16), __uint_as_float(r[1] & 0xffff0000u)};
+                        }
+                    }
+                    a += ys;
+                }
+            }
+            v[j] = a;
+            s += (a[0] + a[1]) + (a[2] + a[3]);
+        }
+        s = wave_sum(s);
+        if (lane == 0) red[0][wave] = s;
+        __syncthreads();
+        const float mean = ((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) / (float)width;
+        float q = 0.f;
+#pragma unroll
+        for (int j = 0; j < V4; ++j) {
+            if (4 * (tid + 256 * j) < width) {
+                const f32x4 d = v[j] - mean;
+                q += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
+            }
+        }
+        q = wave_sum(q);
+        if (lane == 0) red[1][wave] = q;
+        __syncthreads();
+        const float r = 1.0f / sqrtf(((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) / (float)width + eps);
+#pragma unroll
+        for (int j = 0; j < V4; ++j) {
+            const int i = 4 * (tid + 256 * j);
+            if (i < width) {
+                const f32x4 o = (v[j] - mean) * r * *(const f32x4*)(w + i) + *(const f32x4*)(b + i);
+                *(f32x4*)(out + t * width + i) = o;
+                if (cast) {
+                    if (cast_dt == MI355_DT_F32) *(f32x4*)((float*)cast + t * width + i) = o;
+                    else *(u32x2*)((bf16_t*)cast + t * width + i) = u32x2{pack_bf2(o[0], o[1]), pack_bf2(o[2], o[3])};
+                }
+            }
+        }
+        __syncthreads();  // red[] is reused by the next row
+    }
+}
+
 extern "C" int mi355_add_layernorm_fwd(int64_t tokens, int width, const float* x, float alpha, const void* y, int y_dt, int64_t ldy, int parts, const float* w,
                                        const float* b, float eps, float* out, void* cast, int cast_dt, void* stream) {
     MI355_REQUIRE(tokens > 0 && width > 0 && width <= 8192 && x && w && b && out, "add_layernorm_fwd: bad arguments (width <= 8192)");
     MI355_REQUIRE(!y || (dt_ok(y_dt) && parts >= 1 && ldy >= width), "add_layernorm_fwd: bad summand");
     MI355_REQUIRE(!cast || dt_ok(cast_dt), "add_layernorm_fwd: bad cast dtype");
+    const bool aligned = width % 4 == 0 && (!y || (ldy % 4 == 0 && ((uintptr_t)y & 15) == 0)) && ((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
+                         ((uintptr_t)w & 15) == 0 && ((uintptr_t)b & 15) == 0 && (!cast || ((uintptr_t)cast & 15) == 0);
+    if (aligned && width > 512) {
+        const int g = (int)(tokens < 65535 * 8 ? tokens : 65535 * 8);
+#define LNW_CASE(V)                                                                                                                                            \
+    if (width <= 1024 * V) {                                                                                                                                   \
+        add_layernorm_wide_kernel<V><<<g, 256, 0, ST(stream)>>>(tokens, width, x, alpha, y, y_dt, ldy, parts, w, b, eps, out, cast, cast_dt);                \
+        MI355_LAUNCH_CHECK("add_layernorm_fwd");                                                                                                               \
+        return 0;                                                                                                                                              \
+    }
+        LNW_CASE(1) LNW_CASE(2) LNW_CASE(4) LNW_CASE(8)
+#undef LNW_CASE
+    }
     const int grid = rows_grid(tokens, 4);
 #define LN_CASE(E)                                                                                                                                         \
     if (width <= 64 * E) {                                                                                                                                 \
@@ -278,7 +355,7 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 __global__ void gla_kernel(const int* __restrict__ seq_off, const int* __restrict__ slot, int H, int dk, int dv, const void* __restrict__ q, const void* __restrict__ k,
                            const void* __restrict__ v, const void* __restrict__ z, int dt, int z_dt, int64_t ldq, int64_t ldk, int64_t ldv_, int64_t ldz,
                            const float* __restrict__ zbias, float inv_tau, float qscale, float* __restrict__ state, float* __restrict__ o) {
-    extern __shared__ float smem[];
+    extern __shared__ __attribute__((aligned(16))) float smem[];
     const int RC = blockDim.x >> 6;
     float* sq = smem;                       // [TB][dk]
     float* sk = sq + GLA_TB * dk;           // [TB][dk]
@@ -310,17 +387,30 @@ __global__ void gla_kernel(const int* __restrict__ seq_off, const int* __restric
             sv[e] = c < dv ? ld_dt(v, dt, (int64_t)(tb + j) * ldv_ + (int64_t)h * dv + c) : 0.f;
         }
         __syncthreads();
+        const bool full = chunk * GLA_R + GLA_R <= dk && dk % 4 == 0;
         for (int j = 0; j < nt; ++j) {
             const float vv = sv[j * 64 + (threadIdx.x & 63)];
             const float* qa = sq + j * dk + chunk * GLA_R;
             const float* ka = sk + j * dk + chunk * GLA_R;
             const float* aa = sa + j * dk + chunk * GLA_R;
             float acc = 0.f;
+            if (full) {
 #pragma unroll
-            for (int r = 0; r < GLA_R; ++r) {
-                if (chunk * GLA_R + r < dk) {
-                    st[r] = aa[r] * st[r] + ka[r] * vv;
-                    acc += st[r] * qa[r];
+                for (int r4 = 0; r4 < GLA_R / 4; ++r4) {
+                    const f32x4 q4 = *(const f32x4*)(qa + 4 * r4), k4 = *(const f32x4*)(ka + 4 * r4), a4 = *(const f32x4*)(aa + 4 * r4);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        st[4 * r4 + i] = a4[i] * st[4 * r4 + i] + k4[i] * vv;
+                        acc += st[4 * r4 + i] * q4[i];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < GLA_R; ++r) {
+                    if (chunk * GLA_R + r < dk) {
+                        st[r] = aa[r] * st[r] + ka[r] * vv;
+                        acc += st[r] * qa[r];
+                    }
                 }
             }
             sp[(j * RC + chunk) * 64 + (threadIdx.x & 63)] = acc;
@@ -354,6 +444,51 @@ extern "C" int mi355_gla_fwd(int n_seq, const int* seq_off, const int* slot, int
     gla_kernel<<<dim3(n_seq, H, (dv + 63) / 64), 64 * RC, lds_bytes, ST(stream)>>>(seq_off, slot, H, dk, dv, q, k, v, z, dt, z_dt, ldq, ldk, ldv, ldz, zbias, inv_tau, qscale,
                                                                                    state, o);
     MI355_LAUNCH_CHECK("gla_fwd");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------- router logits
+// logits[t, e] = sum_k x[t, k] * W[e, k]: fp32 rows against a small bf16 matrix, fp32 FMA.  One workgroup per token keeps the row in LDS; wave w takes
+// experts w, w + 4, ...; a lane reads 8 weights (16 bytes) at a time when the rows allow it.
+__global__ __launch_bounds__(256) void router_logits_kernel(int64_t T, int E, int Kd, const float* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ W, int64_t ldw,
+                                                            float* __restrict__ out, int vec) {
+    extern __shared__ __attribute__((aligned(16))) float xs[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int64_t t = blockIdx.x; t < T; t += gridDim.x) {
+        __syncthreads();
+        for (int k = tid; k < Kd; k += 256) xs[k] = x[t * ldx + k];
+        __syncthreads();
+        for (int e = wave; e < E; e += 4) {
+            const bf16_t* wr = W + (int64_t)e * ldw;
+            float acc = 0.f;
+            if (vec) {
+                for (int k = lane * 8; k < Kd; k += 512) {
+                    const u32x4 r = *(const u32x4*)(wr + k);
+                    const f32x4 a = *(const f32x4*)(xs + k), c = *(const f32x4*)(xs + k + 4);
+                    acc = fmaf(a[0], __uint_as_float(r[0] << 16), acc);
+                    acc = fmaf(a[1], __uint_as_float(r[0] & 0xffff0000u), acc);
+                    acc = fmaf(a[2], __uint_as_float(r[1] << 16), acc);
+                    acc = fmaf(a[3], __uint_as_float(r[1] & 0xffff0000u), acc);
+                    acc = fmaf(c[0], __uint_as_float(r[2] << 16), acc);
+                    acc = fmaf(c[1], __uint_as_float(r[2] & 0xffff0000u), acc);
+                    acc = fmaf(c[2], __uint_as_float(r[3] << 16), acc);
+                    acc = fmaf(c[3], __uint_as_float(r[3] & 0xffff0000u), acc);
+                }
+            } else {
+                for (int k = lane; k < Kd; k += 64) acc = fmaf(xs[k], bf2f(wr[k]), acc);
+            }
+            acc = wave_sum(acc);
+            if (lane == 0) out[t * E + e] = acc;
+        }
+    }
+}
+
+extern "C" int mi355_router_logits(int64_t tokens, int E, int K, const float* x, int64_t ldx, const void* W, int64_t ldw, float* out, void* stream) {
+    MI355_REQUIRE(tokens > 0 && E > 0 && K > 0 && K <= 16384 && x && W && out && ldx >= K && ldw >= K, "router_logits: bad arguments (width <= 16384)");
+    const int vec = K % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)W & 15) == 0;
+    const int g = (int)(tokens < 65535 * 8 ? tokens : 65535 * 8);
+    router_logits_kernel<<<g, 256, sizeof(float) * K, ST(stream)>>>(tokens, E, K, x, ldx, (const bf16_t*)W, ldw, out, vec);
+    MI355_LAUNCH_CHECK("router_logits");
     return 0;
 }
 

@@ -137,6 +137,17 @@ def gla(q, k, v, z, zbias, inv_tau, qscale, seq_off, slot, state, H, dk, dv):
     return o
 
 
+def router_logits(x32, w):
+    """fp32 [tokens, experts] = x32 (fp32 rows) times w[experts, width]^T (bf16), fp32 FMA."""
+    L.require_gpu(x32, w)
+    _rows(x32, "router_logits(x)")
+    if x32.dtype != F32 or w.dtype != BF16 or w.dim() != 2 or w.stride(1) != 1 or w.shape[1] != x32.shape[1]:
+        raise ValueError("router_logits: x fp32 [tokens, width], w bf16 [experts, width]")
+    out = torch.empty((x32.shape[0], w.shape[0]), dtype=F32, device=x32.device)
+    L.call("mi355_router_logits", x32.shape[0], w.shape[0], w.shape[1], L.ptr(x32), x32.stride(0), L.ptr(w), w.stride(0), L.ptr(out))
+    return out
+
+
 def moe_route(logits, correction, top, groups, keep, scale):
     L.require_gpu(logits, correction)
     if logits.dtype != F32 or not logits.is_contiguous() or (correction is not None and (correction.dtype != F32 or correction.numel() != logits.shape[1])):
@@ -189,8 +200,18 @@ def linear(x, w, out_dtype=None):
     return bgemm(x, w, out, M, N, Kd)
 
 
-def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, desc, max_new, scale):
-    """Two-part-key causal attention over a ragged batch.  ``desc`` = (q_row0, n_new, past, k1_row0, k2_row0, v_row0) int32 [n_seq] each."""
+def attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys):
+    """Workgroups per tile of the MFMA attention: a step with few query tiles and long caches (one-token steps) deals each tile's keys to several, about
+    256 keys each, as many as fill the chip's 256 CUs once."""
+    tiles = n_seq * head_tiles * -(-max_new * hm // 128)
+    if max_keys <= 512 or tiles >= 128:
+        return 1
+    return max(1, min(-(-max_keys // 256), 32, 256 // tiles))
+
+
+def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, desc, max_new, scale, max_keys=0):
+    """Two-part-key causal attention over a ragged batch.  ``desc`` = (q_row0, n_new, past, k1_row0, k2_row0, v_row0) int32 [n_seq] each.  ``max_keys``
+    (the longest sequence's keys, if the caller knows it) lets one-token steps over long caches spread a tile's keys over several workgroups."""
     L.require_gpu(q, k1, k2, v, out, *desc)
     for t, n in ((q, "q"), (k1, "k1"), (v, "v"), (out, "out")):
         _rows(t, f"latent_attn({n})")
@@ -199,6 +220,15 @@ def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, d
     n_seq = desc[0].numel()
     for t in desc:
         _i32(t, "latent_attn(desc)", n_seq)
+    mfma = v.dtype == BF16
+    splits, ws = 1, None
+    if mfma and D1 + D2 <= 320 and DV <= 256 and max_keys:
+        head_tiles = -(-H // hm)
+        splits = attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys)
+        if splits > 1:
+            dvp = 32 if DV <= 32 else 64 if DV <= 64 else 128 if DV <= 128 else 256
+            ws = torch.empty(n_seq * head_tiles * -(-max_new * hm // 128) * splits * 128 * (2 + dvp), dtype=F32, device=v.device)
     L.call("mi355_latent_attn", n_seq, max_new, H, hm, D1, D2, DV, L.ptr(q), q.stride(0), q_hs, L.ptr(k1), k1.stride(0), k1_hs, L.ptr(k2), 0 if k2 is None else k2.stride(0),
-           L.ptr(v), v.stride(0), v_hs, L.ptr(out), out.stride(0), o_hs, _dt(v), *[L.ptr(t) for t in desc], float(scale), 1 if v.dtype == BF16 else 0)
+           L.ptr(v), v.stride(0), v_hs, L.ptr(out), out.stride(0), o_hs, _dt(v), *[L.ptr(t) for t in desc], float(scale), 1 if mfma else 0, splits, L.ptr(ws),
+           0 if ws is None else ws.numel())
     return out

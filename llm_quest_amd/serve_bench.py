@@ -1,0 +1,146 @@
+"""Serving throughput of the registry models with random weights: prompts (one packed step) and one-token steps through the slot cache, beside the
+closest existing model of the package at equal width and depth -- the Qwen3.5 hybrid text stack (gated delta net + gated attention, dense SwiGLU) through
+its own cache.  ``bench.py --serve gemepel`` prints the result as one JSON line; the default workload of ``bench.py`` is untouched.
+
+Sizes resemble real layers (random weights; what is generated means nothing): width 1024 / 2048, 4 layers (three linear-attention layers and one softmax-
+attention layer, as the Qwen3.5 stack has them), 16 experts of which 2 run per token."""
+
+import json
+import time
+
+import torch
+
+BF16 = torch.bfloat16
+
+
+def gemepel_config(width, heads, vocab=32000):
+    lat = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": width // 2, "kv_rank": 256, "rot": {"dims": 64, "base": 1e6}, "scale": 192 ** -0.5}
+    gla = {"heads": 16, "dim": 128, "vdim": 128, "tau": 16.0}
+    mlp = {"kind": "moe", "expert": {"ff": int(width * 1.75)}, "router": {"experts": 16, "top": 2, "groups": {"count": 4, "keep": 2}, "scale": 2.5}}
+    layers = [{"type": "gla", "mixer": gla, "mlp": mlp}, {"type": "gla", "mixer": gla, "mlp": mlp}, {"type": "gla", "mixer": gla, "mlp": mlp},
+              {"type": "latent_attention", "mixer": lat, "mlp": mlp}]
+    return {"architecture": "Gemepel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "postln_alpha": 1.0,
+            "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "layers": layers}
+
+
+def random_gemepel(width, heads, device, decay_rank=64):
+    from llm_quest_amd.gemepel.gemepel_model import GemepelConfig, GemepelModel
+
+    cfg = GemepelConfig(gemepel_config(width, heads))
+    shapes = {f"l{i}.mix.a1": (decay_rank, width) for i in range(len(cfg.layers))}
+    shapes.update({f"l{i}.mlp.correction": (16,) for i in range(len(cfg.layers))})
+    with torch.device(device):
+        model = GemepelModel(cfg, shapes)
+    g = torch.Generator(device=device).manual_seed(7)
+    for name, p in model.named_parameters():
+        if p.dim() >= 2:
+            p.data.copy_((torch.randn(p.shape, device=device, generator=g) / p.shape[-1] ** 0.5).to(BF16))
+        elif name.endswith("_w") or name.endswith("norm"):
+            p.data.fill_(1.0)
+        elif name.endswith("a2_bias"):
+            p.data.fill_(3.0)
+    return model
+
+
+def _time(fn, warmup, steps):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def bench_gemepel(width, heads, batch, prompt, steps, warmup, device):
+    from llm_quest_amd.generate import RaggedBatch
+
+    model = random_gemepel(width, heads, device)
+    vocab = model.vocab_size
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, vocab, (prompt,), generator=g).tolist() for _ in range(batch)]
+    rb = RaggedBatch(model, max_tokens=prompt + steps + warmup + 8, slots=batch)
+    state = {"n": 0}
+
+    def prefill():
+        ids = [(state["n"], i) for i in range(batch)]
+        state["n"] += 1
+        rb.step([(sid, p) for sid, p in zip(ids, prompts)])
+        state["last"] = ids
+
+    def close_last():
+        for sid in state.pop("last", []):
+            rb.finish(sid)
+
+    def prefill_cycle():
+        close_last()
+        prefill()
+
+    t_prefill = _time(prefill_cycle, max(1, warmup // 2), max(2, steps // 8))
+    ids = state["last"]
+    tok = [[5]] * batch
+    t_decode = _time(lambda: rb.step(list(zip(ids, tok))), warmup, steps)
+    close_last()
+    # one sequence alone
+    rb.step([("solo", prompts[0])])
+    t_solo = _time(lambda: rb.step([("solo", [5])]), warmup, steps)
+    params = sum(p.numel() for p in model.parameters())
+    return {"model": f"gemepel-w{width}", "params_M": round(params / 1e6, 1), "prefill_tok_s": round(batch * prompt / t_prefill), "prefill_ms": round(t_prefill * 1e3, 2),
+            "decode_tok_s": round(batch / t_decode), "decode_ms_per_step": round(t_decode * 1e3, 3), "decode_b1_ms_per_step": round(t_solo * 1e3, 3)}
+
+
+def bench_qwen35(width, heads, batch, prompt, steps, warmup, device):
+    from llm_quest_amd.config import QWEN3_5_08B_CONFIG
+    from llm_quest_amd.qwen.qwen3_5.qwen3_5_text_model import Qwen3_5TextModel
+    from llm_quest_amd.utils import Qwen3_5Cache
+
+    cfg = dict(QWEN3_5_08B_CONFIG, vocab_size=32000, emb_dim=width, hidden_dim=int(width * 3.5), n_layers=4, linear_sdpa_ratio=4, n_heads=heads, num_kv_groups=2,
+               context_length=prompt + steps + warmup + 64)
+    torch.manual_seed(3)
+    with torch.device(device):
+        model = Qwen3_5TextModel(cfg).eval()
+    ids = torch.randint(0, 32000, (batch, prompt), device=device)
+    holder = {}
+
+    def prefill():
+        holder["c"] = Qwen3_5Cache(cfg["n_layers"], cfg["linear_sdpa_ratio"], prompt, cfg["context_length"])
+        with torch.inference_mode():
+            model(ids, cache=holder["c"])
+
+    t_prefill = _time(prefill, max(1, warmup // 2), max(2, steps // 8))
+    tok = torch.full((batch, 1), 5, device=device)
+
+    def decode():
+        with torch.inference_mode():
+            model(tok, cache=holder["c"])
+
+    t_decode = _time(decode, warmup, steps)
+    ids1 = ids[:1].contiguous()
+    holder["c"] = Qwen3_5Cache(cfg["n_layers"], cfg["linear_sdpa_ratio"], prompt, cfg["context_length"])
+    with torch.inference_mode():
+        model(ids1, cache=holder["c"])
+    tok1 = tok[:1].contiguous()
+
+    def decode1():
+        with torch.inference_mode():
+            model(tok1, cache=holder["c"])
+
+    t_solo = _time(decode1, warmup, steps)
+    params = sum(p.numel() for p in model.parameters())
+    return {"model": f"qwen3.5-text-w{width}", "params_M": round(params / 1e6, 1), "prefill_tok_s": round(batch * prompt / t_prefill), "prefill_ms": round(t_prefill * 1e3, 2),
+            "decode_tok_s": round(batch / t_decode), "decode_ms_per_step": round(t_decode * 1e3, 3), "decode_b1_ms_per_step": round(t_solo * 1e3, 3)}
+
+
+def run(which, steps, warmup, sizes=((1024, 8), (2048, 16)), batch=8, prompt=1024, device="cuda", with_reference=True):
+    if which != "gemepel":
+        raise SystemExit(f"--serve: unknown model {which!r}")
+    rows = []
+    for width, heads in sizes:
+        rows.append(bench_gemepel(width, heads, batch, prompt, steps, warmup, device))
+        if with_reference:
+            rows.append(bench_qwen35(width, heads, batch, prompt, steps, warmup, device))
+    out = {"metric": "serving throughput (random weights)", "unit": "tokens/s", "batch": batch, "prompt": prompt, "steps": steps, "warmup": warmup,
+           "dtype": "bf16", "data": "synthetic", "rows": rows}
+    print(json.dumps(out))
+    return out

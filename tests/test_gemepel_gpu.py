@@ -310,6 +310,34 @@ def test_attention_finds_one_far_key_among_hundreds(dt, far):
     assert rel(out.view(3, H, D1)[-1], ks[far].expand(H, D1)) < 0.05
 
 
+@pytest.mark.parametrize("far", [0, 255, 256, 1023, 1024, 1499])
+def test_attention_with_the_keys_dealt_to_several_workgroups(far):
+    """One-token steps over a long cache: each tile's keys are split over workgroups and joined afterwards.  Two sequences of different lengths share the
+    step; the far key of the longer one lies in the first, a middle or the last share, and at the shares' borders."""
+    from llm_quest_amd import kernels_seq as S
+
+    H, D1, D2, L, L2 = 5, 40, 16, 1500, 333
+    g = torch.Generator().manual_seed(far)
+    rows = torch.randn(L + L2, D1 + D2, generator=g).to(BF16)
+    kf = rows.float()
+    qs = torch.randn(2, H, D1 + D2, generator=g)
+    qs[0] = 3.0 * kf[far]
+    scale = 0.25
+    want = []
+    for n, (lo, hi) in enumerate(((0, L), (L, L + L2))):
+        k = kf[lo:hi]
+        want.append(_attention_reference(qs[n : n + 1].double(), k[:, None, :D1].expand(-1, H, -1).double(), k[:, D1:].double(), k[:, None, :D1].expand(-1, H, -1).double(),
+                                         hi - lo - 1, scale)[0])
+    out = torch.empty(2, H * D1, dtype=BF16, device=DEV)
+    dr = rows.to(DEV)
+    starts = dev_i32([0, L])
+    S.latent_attn(qs.view(2, -1).to(DEV), dr, dr[:, D1:], dr, out, H, 8, D1, D2, D1, D1 + D2, 0, 0, D1, (dev_i32([0, 1]), dev_i32([1, 1]), dev_i32([L - 1, L2 - 1]), starts, starts, starts),
+                  1, scale, max_keys=L)
+    assert S.attn_key_splits(2, 1, 1, 8, L) > 1
+    assert rel(out.view(2, H, D1), torch.stack(want)) < 2e-2
+    assert rel(out.view(2, H, D1)[0], kf[far, :D1].expand(H, D1)) < 0.05
+
+
 @pytest.mark.parametrize("dt", [F32, BF16])
 def test_gla_kernel_carries_state_over_cuts_and_keeps_a_far_token(dt):
     from llm_quest_amd import kernels_seq as S
