@@ -204,6 +204,121 @@ __global__ __launch_bounds__(256) void bgemm_mfma_kernel(BgemmArgs p) {
         }
 }
 
+// ---- MFMA path, 128 x 128 tile: four waves of 64 x 64 (2 x 2 blocks of 32 x 32), k in steps of 32; the next step's operands are fetched into registers
+// while the current step multiplies from LDS (one LDS stage, two barriers per step).  Four LDS fragment reads feed four MFMAs.
+#define TM 128
+__global__ __launch_bounds__(256) void bgemm_mfma128_kernel(BgemmArgs p) {
+    __shared__ __attribute__((aligned(16))) bf16_t As[TM][MK + MPAD];
+    __shared__ __attribute__((aligned(16))) bf16_t Bs[TM][MK + MPAD];
+    const int b = blockIdx.z;
+    int row0 = 0, rows = p.M;
+    if (p.grp_offs) {
+        row0 = p.grp_offs[b];
+        rows = p.grp_offs[b + 1] - row0;
+    }
+    const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TM;
+    if (m0 >= rows) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, ln = lane & 31, hf = lane >> 5;
+    const bf16_t* A = (const bf16_t*)p.A;
+    const bf16_t* B = (const bf16_t*)p.B;
+    const bool b_kfast = p.sbk == 1;
+    const int64_t b_base = (int64_t)b * p.b_bs;
+    const bool a_vec = (p.lda % 8 == 0) && (p.a_bs % 8 == 0) && (((uintptr_t)p.A & 15) == 0);
+    const bool b_vec = b_kfast && (p.sbn % 8 == 0) && (p.b_bs % 8 == 0) && (((uintptr_t)p.B & 15) == 0);
+    // loader roles: chunk c = tid + 256 i (i < 2): row c / 4, k offset (c % 4) * 8
+    int64_t a_base[2];
+    int lr[2], lk[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int c = tid + 256 * i;
+        lr[i] = c >> 2, lk[i] = (c & 3) * 8;
+        a_base[i] = -1;
+        if (m0 + lr[i] < rows) {
+            const int r = row0 + m0 + lr[i];
+            const int64_t arow = p.a_rows ? p.a_rows[r] / p.a_div : r;
+            a_base[i] = (int64_t)b * p.a_bs + arow * p.lda;
+        }
+    }
+    u32x4 ra[2], rb[2];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            u32x4 va = {0u, 0u, 0u, 0u}, vb = {0u, 0u, 0u, 0u};
+            if (a_base[i] >= 0) {
+                if (a_vec && k0 + lk[i] + 8 <= p.K) va = *(const u32x4*)(A + a_base[i] + k0 + lk[i]);
+                else {
+                    bf16_t e[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) e[j] = k0 + lk[i] + j < p.K ? A[a_base[i] + k0 + lk[i] + j] : (bf16_t)0;
+                    va = u32x4{(unsigned)e[0] | ((unsigned)e[1] << 16), (unsigned)e[2] | ((unsigned)e[3] << 16), (unsigned)e[4] | ((unsigned)e[5] << 16), (unsigned)e[6] | ((unsigned)e[7] << 16)};
+                }
+            }
+            const int n = n0 + lr[i];
+            if (n < p.N) {
+                if (b_vec && k0 + lk[i] + 8 <= p.K) vb = *(const u32x4*)(B + b_base + (int64_t)n * p.sbn + k0 + lk[i]);
+                else {
+                    bf16_t e[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) e[j] = k0 + lk[i] + j < p.K ? B[b_base + (int64_t)n * p.sbn + (int64_t)(k0 + lk[i] + j) * p.sbk] : (bf16_t)0;
+                    vb = u32x4{(unsigned)e[0] | ((unsigned)e[1] << 16), (unsigned)e[2] | ((unsigned)e[3] << 16), (unsigned)e[4] | ((unsigned)e[5] << 16), (unsigned)e[6] | ((unsigned)e[7] << 16)};
+                }
+            }
+            ra[i] = va, rb[i] = vb;
+        }
+    };
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    fetch(0);
+    for (int k0 = 0; k0 < p.K; k0 += MK) {
+        __syncthreads();  // the previous step's fragments are read
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            *(u32x4*)&As[lr[i]][lk[i]] = ra[i];
+            *(u32x4*)&Bs[lr[i]][lk[i]] = rb[i];
+        }
+        __syncthreads();
+        if (k0 + MK < p.K) fetch(k0 + MK);
+#pragma unroll
+        for (int kk = 0; kk < MK; kk += 8) {
+            const bf16x4 a0 = *(const bf16x4*)&As[wm + ln][kk + 4 * hf], a1 = *(const bf16x4*)&As[wm + 32 + ln][kk + 4 * hf];
+            const bf16x4 b0 = *(const bf16x4*)&Bs[wn + ln][kk + 4 * hf], b1 = *(const bf16x4*)&Bs[wn + 32 + ln][kk + 4 * hf];
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a1, b1, acc[1][1], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int m = m0 + wm + 32 * bi + 8 * g + 4 * hf + i;
+                if (m >= rows) continue;
+                const int r = row0 + m;
+                const int64_t crow = p.c_rows ? p.c_rows[r] : r;
+                const float sc = p.row_scale ? p.row_scale[crow] : 1.0f;
+                const int64_t cb = (int64_t)b * p.c_bs + crow * p.ldc;
+#pragma unroll
+                for (int bj = 0; bj < 2; ++bj) {
+                    const int n = n0 + wn + 32 * bj + ln;
+                    if (n >= p.N) continue;
+                    float v = acc[bi][bj][4 * g + i];
+                    if (p.epi == 1) v = v > 0.f ? v * v : 0.f;
+                    v *= sc;
+                    if (p.c_dt == MI355_DT_F32) ((float*)p.C)[cb + n] = v;
+                    else ((bf16_t*)p.C)[cb + n] = f2bf(v);
+                }
+            }
+}
+
 extern "C" int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t lda, int64_t a_bs, const void* B, int b_dt, int64_t sbn, int64_t sbk,
                            int64_t b_bs, void* C, int c_dt, int64_t ldc, int64_t c_bs, const int* grp_offs, const int* a_rows, int a_div, const int* c_rows,
                            const float* row_scale, int epi, int use_mfma, void* stream) {
@@ -220,6 +335,13 @@ extern "C" int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_
     p.M = M, p.N = N, p.K = K;
     p.grp_offs = grp_offs, p.a_rows = a_rows, p.a_div = a_rows ? a_div : 1, p.c_rows = c_rows, p.row_scale = row_scale;
     p.epi = epi, p.a_dt = a_dt, p.b_dt = b_dt, p.c_dt = c_dt;
+    if (use_mfma && sbk == 1 && N >= 128 && K >= 64) {  // the large tile: weights stored [out, in], enough columns to fill it
+        const int64_t my128 = ((int64_t)M + TM - 1) / TM;
+        MI355_REQUIRE(my128 <= 65535, "bgemm: too many row tiles");
+        bgemm_mfma128_kernel<<<dim3((N + TM - 1) / TM, (unsigned)my128, batch), 256, 0, ST(stream)>>>(p);
+        MI355_LAUNCH_CHECK("bgemm");
+        return 0;
+    }
     const int64_t my = ((int64_t)M + BM - 1) / BM;
     MI355_REQUIRE(my <= 65535, "bgemm: too many row tiles");
     const dim3 grid((N + BN - 1) / BN, (unsigned)my, batch);
