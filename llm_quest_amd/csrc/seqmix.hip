@@ -372,21 +372,53 @@ __global__ void gla_kernel(const int* __restrict__ seq_off, const int* __restric
         const int i = chunk * GLA_R + r;
         st[r] = (col_ok && i < dk) ? S[(int64_t)i * dv + col] : 0.f;
     }
+    // the next group's rows travel from memory into registers while the current group is worked on (a group's loads would otherwise cost a full
+    // memory round trip between every eight tokens); dk <= 16 RC, so a thread carries at most 2 entries of q / k / z and 8 of v
+    float rq[2], rk[2], rz[2], rv[8];
+    auto fetch = [&](int tb) {
+        const int nt = min(GLA_TB, t1 - tb);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int e = threadIdx.x + u * blockDim.x;
+            rq[u] = rk[u] = rz[u] = 0.f;
+            if (e < nt * dk) {
+                const int j = e / dk, i = e % dk;
+                const int64_t t = tb + j;
+                rq[u] = ld_dt(q, dt, t * ldq + (int64_t)h * dk + i);
+                rk[u] = ld_dt(k, dt, t * ldk + (int64_t)h * dk + i);
+                rz[u] = ld_dt(z, z_dt, t * ldz + (int64_t)h * dk + i) + zbias[h * dk + i];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int e = threadIdx.x + u * blockDim.x;
+            rv[u] = 0.f;
+            if (e < nt * 64) {
+                const int j = e >> 6, c = blockIdx.z * 64 + (e & 63);
+                if (c < dv) rv[u] = ld_dt(v, dt, (int64_t)(tb + j) * ldv_ + (int64_t)h * dv + c);
+            }
+        }
+    };
+    if (t0 < t1) fetch(t0);
     for (int tb = t0; tb < t1; tb += GLA_TB) {
         const int nt = min(GLA_TB, t1 - tb);
-        __syncthreads();  // the previous group's partial sums are consumed
-        for (int e = threadIdx.x; e < nt * dk; e += blockDim.x) {
-            const int j = e / dk, i = e % dk;
-            const int64_t t = tb + j;
-            sq[j * dk + i] = ld_dt(q, dt, t * ldq + (int64_t)h * dk + i) * qscale;
-            sk[j * dk + i] = ld_dt(k, dt, t * ldk + (int64_t)h * dk + i);
-            sa[j * dk + i] = expf(inv_tau * log_sigmoid(ld_dt(z, z_dt, t * ldz + (int64_t)h * dk + i) + zbias[h * dk + i]));
+        __syncthreads();  // the previous group's rows and partial sums are consumed
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int e = threadIdx.x + u * blockDim.x;
+            if (e < nt * dk) {
+                sq[e] = rq[u] * qscale;
+                sk[e] = rk[u];
+                sa[e] = expf(inv_tau * log_sigmoid(rz[u]));
+            }
         }
-        for (int e = threadIdx.x; e < nt * 64; e += blockDim.x) {
-            const int j = e >> 6, c = blockIdx.z * 64 + (e & 63);
-            sv[e] = c < dv ? ld_dt(v, dt, (int64_t)(tb + j) * ldv_ + (int64_t)h * dv + c) : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int e = threadIdx.x + u * blockDim.x;
+            if (e < nt * 64) sv[e] = rv[u];
         }
         __syncthreads();
+        if (tb + GLA_TB < t1) fetch(tb + GLA_TB);
         const bool full = chunk * GLA_R + GLA_R <= dk && dk % 4 == 0;
         for (int j = 0; j < nt; ++j) {
             const float vv = sv[j * 64 + (threadIdx.x & 63)];
