@@ -50,12 +50,12 @@ class GemepelBlock(nn.Module):
             src = m.get("kv_from")
             if src is not None and not (0 <= src < i and cfg.layers[src]["type"] == "latent_attention" and cfg.layers[src]["mixer"].get("kv_from") is None):
                 raise ValueError(f"layer {i}: kv_from must name an earlier latent-attention layer with key/value rows of its own")
-            rot = m.get("rot") or {"dims": m["rot_dim"], "base": 10000.0}
-            if src is not None:
-                sm = cfg.layers[src]["mixer"]
-                if (sm["kv_rank"], sm["rot_dim"], sm.get("rot")) != (m["kv_rank"], m["rot_dim"], m.get("rot")):
+            sm = cfg.layers[src]["mixer"] if src is not None else None
+            rot = m.get("rot") or (sm.get("rot") if sm else None) or {"dims": m["rot_dim"], "base": 10000.0}
+            if sm is not None:
+                if (sm["kv_rank"], sm["rot_dim"]) != (m["kv_rank"], m["rot_dim"]) or (sm.get("rot") and m.get("rot") and sm["rot"] != m["rot"]):
                     raise ValueError(f"layer {i}: kv_from = {src} needs that layer's kv_rank, rot_dim and rotation to equal this layer's")
-            self.mixer = LatentAttention(w, m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["q_rank"], m["kv_rank"], m["scale"], rot["dims"], rot["base"], cfg.eps, i, kv_from=src)
+            self.mixer = LatentAttention(w, m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["q_rank"], m["kv_rank"], m.get("scale", (m["dim"] + m["rot_dim"]) ** -0.5), rot["dims"], rot["base"], cfg.eps, i, kv_from=src)
         else:
             self.mixer = GatedLinearAttention(w, m["heads"], m["dim"], m["vdim"], shapes[f"l{i}.mix.a1"][0], m["tau"], cfg.eps, i)
         self.norm1_w, self.norm1_b = nn.Parameter(torch.ones(w, dtype=BF16), requires_grad=False), nn.Parameter(torch.zeros(w, dtype=BF16), requires_grad=False)

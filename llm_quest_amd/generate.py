@@ -183,7 +183,8 @@ class RaggedBatch:
     def __init__(self, model, max_tokens=0, slots=4, device=None):
         self.model = model
         self.device = device or next(model.parameters()).device
-        self.cache = model.new_cache(self.device, max_tokens=max_tokens, slots=slots)
+        # max_tokens is a hint for the rows a slot starts with (rows grow on demand, so a generous hint must not reserve slots x hint rows up front)
+        self.cache = model.new_cache(self.device, max_tokens=min(int(max_tokens), 8192), slots=slots)
 
     def step(self, entries, want=None, return_layers=False):
         """entries: [(seq_id, [token, ...])] in batch order.  want: per entry the positions among ITS new tokens whose logits are asked for (default:
@@ -218,7 +219,8 @@ class RaggedBatch:
         return out if rows else None
 
     def finish(self, seq_id):
-        self.cache.close(seq_id)
+        if seq_id in self.cache:
+            self.cache.close(seq_id)
 
 
 def generate_ragged(model, prompts, max_gen, top_k=None, top_p=None, min_p=None, temp=0.0, eos_ids=None, max_tokens=0):
