@@ -24,31 +24,40 @@ class SeqStep:
 
     def __init__(self, cache, entries, device, act_dtype):
         self.cache, self.act_dtype, self.device = cache, act_dtype, device
-        tok, prev, pos, seq_off, slots, past, n_new = [], [], [], [0], [], [], []
+        import numpy as np
+
+        seq_off, slots, past, n_new = [0], [], [], []
         for slot, new in entries:
             if len(new) == 0:
                 raise ValueError("SeqStep: a sequence of the step brings no token")
-            start = cache.length[slot]
-            tok.extend(new)
-            prev.append(cache.last_token[slot])
-            prev.extend(new[:-1])
-            pos.extend(range(start, start + len(new)))
             seq_off.append(seq_off[-1] + len(new))
             slots.append(slot)
-            past.append(start)
+            past.append(cache.length[slot])
             n_new.append(len(new))
         cache.reserve(max(p + n for p, n in zip(past, n_new)))
         cap = cache.capacity
-        self.T, self.n_seq, self.max_new = len(tok), len(slots), max(n_new)
+        self.T, self.n_seq, self.max_new = seq_off[-1], len(slots), max(n_new)
         self.max_keys = max(p + n for p, n in zip(past, n_new))
         self.fresh = all(p == 0 for p in past)
         self.host_seq_off = seq_off
-        row0 = [s * cap for s in slots]
-        dst = [row0[i] + p for i in range(len(slots)) for p in range(past[i], past[i] + n_new[i])]
-        # one host-to-device copy for all descriptors
-        flat = tok + prev + pos + dst + seq_off + slots + past + n_new + row0 + list(range(self.T))
-        buf = torch.tensor(flat, dtype=I32).to(device, non_blocking=False)
         T, n = self.T, self.n_seq
+        row0 = [s * cap for s in slots]
+        # rows of the descriptor block: tokens | previous token | position | cache row | per-sequence arrays | 0 .. T-1; one host-to-device copy for all
+        buf = np.empty(5 * T + 5 * n + 1, dtype=np.int32)
+        tok, prev, pos, dst = buf[0:T], buf[T : 2 * T], buf[2 * T : 3 * T], buf[3 * T : 4 * T]
+        for i, (slot, new) in enumerate(entries):
+            a, b = seq_off[i], seq_off[i + 1]
+            tok[a:b] = new
+            prev[a] = cache.last_token[slot]
+            prev[a + 1 : b] = tok[a : b - 1]
+            pos[a:b] = np.arange(past[i], past[i] + n_new[i], dtype=np.int32)
+            dst[a:b] = pos[a:b] + row0[i]
+        at = 4 * T
+        for arr in (seq_off, slots, past, n_new, row0):
+            buf[at : at + len(arr)] = arr
+            at += len(arr)
+        buf[at : at + T] = np.arange(T, dtype=np.int32)
+        buf = torch.from_numpy(buf).to(device, non_blocking=False)
         cuts = [T, T, T, T, n + 1, n, n, n, n, T]
         parts, at = [], 0
         for c in cuts:

@@ -195,9 +195,11 @@ class RaggedBatch:
             return None
         cache, vocab = self.cache, self.model.vocab_size
         slotted = []
+        import numpy as np
+
         for seq_id, toks in entries:
-            toks = [int(t) for t in toks]
-            if any(t < 0 or t >= vocab for t in toks):
+            toks = np.asarray(toks, dtype=np.int64).reshape(-1)
+            if toks.size and (int(toks.min()) < 0 or int(toks.max()) >= vocab):
                 raise ValueError(f"sequence {seq_id!r}: token id outside [0, {vocab})")
             slot = cache.slot(seq_id) if seq_id in cache else cache.open(seq_id)
             slotted.append((slot, toks))
