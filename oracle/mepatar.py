@@ -1,0 +1,206 @@
+"""Plain PyTorch-CPU oracle of the Mepatar decoder (test infrastructure only, one function per mechanism).
+
+Mepatar is a pre-norm decoder with PARALLEL sublayers: x <- x + mixer(n1(x)) + ff(n2(x)), both norms of the same x.  The norms are RMS norms taken
+over equal consecutive groups of the row.  What a mixer reads first passes a short causal convolution over time that is added to it (h + conv(h)).
+Mixers: *retention* (linear attention with one fixed decay per head, rotate-half rotary), *attention* (grouped queries, query / key norm, interleaved
+rotary, a per-head temperature, sliding window that also keeps the first tokens), *delta* (gated delta rule behind short convolutions).  Feed-forward:
+a dense GELU-gated layer or a softmax-routed mixture of clamped gated experts.
+
+Everything here works on ONE whole sequence, in the dtype of the tensors handed in (fp32 or fp64), token by token where a recurrence is involved, and
+shares no code with ``llm_quest_amd``.  ``weights`` maps the checkpoint's tensor names to tensors; ``cfg`` is the parsed ``config.json``.
+"""
+
+import math
+
+import torch
+
+
+def group_rms_norm(x, w, groups, eps):
+    """x [T, n]: every one of ``groups`` equal consecutive parts divided by its own root mean square, the whole times w."""
+    T, n = x.shape
+    p = x.reshape(T, groups, n // groups)
+    p = p / torch.sqrt((p * p).mean(dim=-1, keepdim=True) + eps)
+    return p.reshape(T, n) * w
+
+
+def unit_rms(x, eps):
+    return x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps)
+
+
+def gelu_tanh(z):
+    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+
+
+def silu(z):
+    return z * torch.sigmoid(z)
+
+
+def causal_conv(h, w):
+    """h [T, C], w [C, taps]: y_t = sum_j w[:, j] h_(t - taps + 1 + j), zeros before the first token (the last column weighs the current token)."""
+    T, C = h.shape
+    taps = w.shape[1]
+    y = torch.zeros_like(h)
+    for t in range(T):
+        for j in range(taps):
+            s = t - taps + 1 + j
+            if s >= 0:
+                y[t] += w[:, j] * h[s]
+    return y
+
+
+def rotary(x, dims, base, layout):
+    """x [T, H, D], positions 0 .. T-1.  The first ``dims`` entries of every head turn: pair i is (i, i + dims/2) in the 'half' layout and (2i, 2i+1)
+    in the 'interleaved' one; angle = position * base^(-2i/dims)."""
+    T = x.shape[0]
+    half = dims // 2
+    out = x.clone()
+    for i in range(half):
+        a, b = (i, i + half) if layout == "half" else (2 * i, 2 * i + 1)
+        f = base ** (-2.0 * i / dims)
+        ang = torch.arange(T, dtype=x.dtype) * f
+        c, s = torch.cos(ang)[:, None], torch.sin(ang)[:, None]
+        u, v = x[:, :, a], x[:, :, b]
+        out[:, :, a] = u * c - v * s
+        out[:, :, b] = v * c + u * s
+    return out
+
+
+def retention(q, k, v, decay):
+    """q, k [T, H, dk], v [T, H, dv], decay [H]: S_t = decay S_(t-1) + k_t v_t^T, o_t = S_t^T q_t."""
+    T, H, dk = q.shape
+    dv = v.shape[-1]
+    out = torch.zeros(T, H, dv, dtype=q.dtype)
+    for h in range(H):
+        S = torch.zeros(dk, dv, dtype=q.dtype)
+        for t in range(T):
+            S = decay[h] * S + torch.outer(k[t, h], v[t, h])
+            out[t, h] = S.T @ q[t, h]
+    return out
+
+
+def retention_mixer(h, w, pre, m, eps):
+    T = h.shape[0]
+    H, dk, dv = m["heads"], m["dim"], m["vdim"]
+    q = (h @ w[pre + "q"].T).reshape(T, H, dk)
+    k = (h @ w[pre + "k"].T).reshape(T, H, dk)
+    v = (h @ w[pre + "v"].T).reshape(T, H, dv)
+    q = rotary(q, m["rot"]["dims"], m["rot"]["base"], "half")
+    k = rotary(k, m["rot"]["dims"], m["rot"]["base"], "half") * dk ** -0.5
+    o = retention(q, k, v, [float(d) for d in m["decay"]])
+    o = unit_rms(o, eps).reshape(T, H * dv) * silu(h @ w[pre + "g"].T)
+    return o @ w[pre + "o"].T
+
+
+def visible(i, j, size, keep_first):
+    return j <= i and (i - j < size or j < keep_first)
+
+
+def window_attention(q, k, v, scale, temp, size, keep_first):
+    """q [T, H, d], k [T, G, d], v [T, G, dv]; query head h reads key/value head h // (H/G); softmax over the visible keys."""
+    T, H, d = q.shape
+    G, dv = k.shape[1], v.shape[-1]
+    out = torch.zeros(T, H, dv, dtype=q.dtype)
+    for h in range(H):
+        g = h // (H // G)
+        for i in range(T):
+            js = [j for j in range(i + 1) if visible(i, j, size, keep_first)]
+            s = torch.stack([(q[i, h] * k[j, g]).sum() for j in js]) * scale * temp[h]
+            p = torch.softmax(s, dim=0)
+            out[i, h] = (p[:, None] * torch.stack([v[j, g] for j in js])).sum(dim=0)
+    return out
+
+
+def attention_mixer(h, w, pre, m, eps):
+    T = h.shape[0]
+    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    q = (h @ w[pre + "q"].T + w[pre + "q.b"]).reshape(T, H, d)
+    k = (h @ w[pre + "k"].T + w[pre + "k.b"]).reshape(T, G, d)
+    v = (h @ w[pre + "v"].T + w[pre + "v.b"]).reshape(T, G, dv)
+    q = unit_rms(q, eps) * w[pre + "q.norm"]
+    k = unit_rms(k, eps) * w[pre + "k.norm"]
+    q = rotary(q, m["rot"]["dims"], m["rot"]["base"], "interleaved")
+    k = rotary(k, m["rot"]["dims"], m["rot"]["base"], "interleaved")
+    o = window_attention(q, k, v, m["scale"], w[pre + "temp"], m["mask"]["size"], m["mask"]["keep_first"])
+    return o.reshape(T, H * dv) @ w[pre + "o"].T + w[pre + "o.b"]
+
+
+def delta_rule(q, k, v, beta, g):
+    """q, k [T, H, dk] (already one per value head), v [T, H, dv], beta, g [T, H]: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q."""
+    T, H, dk = q.shape
+    dv = v.shape[-1]
+    out = torch.zeros(T, H, dv, dtype=q.dtype)
+    for h in range(H):
+        S = torch.zeros(dk, dv, dtype=q.dtype)
+        for t in range(T):
+            S = g[t, h] * S
+            u = beta[t, h] * (v[t, h] - S.T @ k[t, h])
+            S = S + torch.outer(k[t, h], u)
+            out[t, h] = S.T @ q[t, h]
+    return out
+
+
+def delta_mixer(h, w, pre, m, eps):
+    T = h.shape[0]
+    H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    q = silu(causal_conv(h @ w[pre + "q"].T, w[pre + "q.conv"])).reshape(T, G, dk)
+    k = silu(causal_conv(h @ w[pre + "k"].T, w[pre + "k.conv"])).reshape(T, G, dk)
+    v = silu(causal_conv(h @ w[pre + "v"].T, w[pre + "v.conv"])).reshape(T, H, dv)
+    q = q / torch.sqrt((q * q).sum(dim=-1, keepdim=True) + 1e-6) * dk ** -0.5
+    k = k / torch.sqrt((k * k).sum(dim=-1, keepdim=True) + 1e-6)
+    rep = H // G
+    q, k = q.repeat_interleave(rep, dim=1), k.repeat_interleave(rep, dim=1)
+    beta = torch.sigmoid(h @ w[pre + "b"].T)
+    g = torch.exp(-torch.exp(w[pre + "A_log"]) * torch.nn.functional.softplus(h @ w[pre + "a"].T + w[pre + "dt_bias"]))
+    o = delta_rule(q, k, v, beta, g)
+    o = (unit_rms(o, eps) * w[pre + "norm"]).reshape(T, H * dv) * silu(h @ w[pre + "g"].T)
+    return o @ w[pre + "o"].T
+
+
+def dense_ff(h, w, pre):
+    return (gelu_tanh(h @ w[pre + "gate"].T) * (h @ w[pre + "up"].T)) @ w[pre + "down"].T
+
+
+def expert_ff(h, w, pre, limit):
+    g = torch.clamp(h @ w[pre + "gate"].T, max=limit)
+    u = torch.clamp(h @ w[pre + "up"].T, min=-limit, max=limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w[pre + "down"].T
+
+
+def route(h, w_router, top):
+    """(chosen experts [T, top], their weights [T, top]): softmax over ALL experts, the ``top`` largest scores, not renormalised."""
+    s = torch.softmax(h @ w_router.T, dim=-1)
+    wts, ids = torch.topk(s, top, dim=-1)
+    return ids, wts
+
+
+def moe_ff(h, w, pre, mlp):
+    ids, wts = route(h, w[pre + "router"], mlp["router"]["top"])
+    out = torch.zeros_like(h)
+    for t in range(h.shape[0]):
+        for e, a in zip(ids[t].tolist(), wts[t]):
+            out[t] += a * expert_ff(h[t : t + 1], w, f"{pre}e{e}.", mlp["expert"]["limit"])[0]
+    return out
+
+
+MIXERS = {"retention": retention_mixer, "attention": attention_mixer, "delta": delta_mixer}
+
+
+def forward(tokens, weights, cfg, dtype=torch.float64, return_layers=False):
+    """tokens: the ids of one whole sequence -> logits [T, vocab] (and the residual stream after every layer)."""
+    w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
+    eps, groups = cfg["norm"]["eps"], cfg["norm"]["groups"]
+    x = w["embed"][torch.tensor(list(tokens))] * cfg["embedding"]["scale"]
+    layers = []
+    for i, layer in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        h1 = group_rms_norm(x, w[p + "norm1"], groups, eps)
+        h1 = h1 + causal_conv(h1, w[p + "canon1"])
+        y = MIXERS[layer["type"]](h1, w, p + "mix.", layer["mixer"], eps)
+        mlp = layer.get("mlp")
+        if mlp is not None:
+            h2 = group_rms_norm(x, w[p + "norm2"], groups, eps)
+            y = y + (dense_ff(h2, w, p + "mlp.") if mlp["kind"] == "dense" else moe_ff(h2, w, p + "mlp.", mlp))
+        x = x + y
+        layers.append(x)
+    logits = group_rms_norm(x, w["final.norm"], groups, eps) @ w["head"].T
+    return (logits, layers) if return_layers else logits
