@@ -524,42 +524,77 @@ int mi355_rmsnorm_rows(int64_t tokens, int n, const void* x, int x_dt, int64_t l
 int mi355_latent_kv_append(int64_t tokens, int rank, int rot, const void* src, int src_dt, int64_t ld, const float* w, float eps, const int* pos,
                            const int* dst_row, const float* freq, int dims, void* cache, int cache_dt, int64_t ldc, void* stream);
 /* dst[t, h * dst_hs + dst_off + i] = src[t, h * src_hs + src_off + i] for i < n (dst fp32), the pairs of [rot_start, rot_start + dims) turned by
- * pos[t] * freq[i] (interleaved rotary embedding). */
+ * pos[t] * freq[i].  layout 0: pair i = entries (2i, 2i+1) (interleaved rotary embedding); layout 1: pair i = entries (i, i + dims/2) (rotate-half). */
 int mi355_rope_heads(int64_t tokens, int H, int n, const void* src, int src_dt, int64_t ld_src, int src_hs, int src_off, float* dst, int64_t ld_dst,
-                     int dst_hs, int dst_off, int rot_start, int dims, const float* freq, const int* pos, void* stream);
+                     int dst_hs, int dst_off, int rot_start, int dims, int layout, const float* freq, const int* pos, void* stream);
 /* out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * w * silu(gate[t, h, :]); o fp32 [tokens, H * D], w fp32 [D]. */
 int mi355_gated_headnorm(int64_t tokens, int H, int D, const float* o, const float* w, const void* gate, int g_dt, int64_t ldg, float eps, void* out,
                          int out_dt, int64_t ldo, void* stream);
 /* Gated linear attention over the rows [seq_off[s], seq_off[s+1]) of each sequence s, state[slot[s]] (fp32 [H, dk, dv]) read and written:
  * S <- diag(a_t) S + k_t v_t^T, o_t = S^T (q_t * qscale), a_t = sigmoid(z_t + zbias)^inv_tau.  q / k rows [H * dk], v rows [H * dv] of dtype dt, z rows [H * dk] of dtype z_dt,
- * o fp32 [tokens, H * dv].  dk <= 256. */
+ * o fp32 [tokens, H * dv].  dk <= 256.  head_decay (fp32 [H], may be NULL): if given, a_t = head_decay[h] for every key channel of head h (retention with a
+ * fixed decay per head; z and zbias may then be NULL).  k_t is multiplied by kscale before it enters the state. */
 int mi355_gla_fwd(int n_seq, const int* seq_off, const int* slot, int H, int dk, int dv, const void* q, const void* k, const void* v, const void* z, int dt,
-                  int z_dt, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldz, const float* zbias, float inv_tau, float qscale, float* state, float* o, void* stream);
+                  int z_dt, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldz, const float* zbias, float inv_tau, float qscale, const float* head_decay,
+                  float kscale, float* state, float* o, void* stream);
 /* logits[t, e] = sum_k x[t, k] W[e, k]: fp32 rows (pitch ldx) against a bf16 matrix [E, K] (pitch ldw), fp32 FMA; out fp32 [tokens, E]. */
 int mi355_router_logits(int64_t tokens, int E, int K, const float* x, int64_t ldx, const void* W, int64_t ldw, float* out, void* stream);
 /* Grouped sigmoid router: s = sigmoid(logits), choice = s + correction (may be NULL); a group (E / groups neighbours) scores the sum of its two
  * largest choices, experts outside the `keep` best groups are excluded, the `top` largest choices win; wts = s / (sum + 1e-20) * scale.
- * ids int32 [tokens, top] in descending order of choice, wts fp32 [tokens, top]. */
-int mi355_moe_route(int64_t tokens, int E, int top, int groups, int keep, const float* logits, const float* correction, float scale, int* ids, float* wts,
-                    void* stream);
+ * ids int32 [tokens, top] in descending order of choice, wts fp32 [tokens, top].  mode 1 (softmax router): s = softmax(logits) over all experts, the `top`
+ * largest win, wts = their s * scale without renormalisation (correction / groups unused). */
+int mi355_moe_route(int64_t tokens, int E, int top, int groups, int keep, const float* logits, const float* correction, float scale, int mode, int* ids,
+                    float* wts, void* stream);
 /* Dispatch lists of `entries` = tokens * top choices: offs int32 [E + 1], perm int32 [entries] = the entries sorted by expert (token order inside one). */
 int mi355_moe_dispatch(int64_t entries, int E, const int* ids, int* offs, int* perm, void* stream);
 /* C[b][m, n] = epi(sum_k A[b][m, k] B[b][n, k]) with general strides: A at b * a_bs + row * lda + k, B at b * b_bs + n * sbn + k * sbk (one of sbn / sbk
  * is 1), C at b * c_bs + row * ldc + n.  grp_offs (may be NULL): batch b owns the sorted rows [grp_offs[b], grp_offs[b+1]) and M bounds their number;
  * a_rows: sorted row r reads A row a_rows[r] / a_div; c_rows: it writes C row c_rows[r]; row_scale: that C row is scaled.  epi 1 = relu(x)^2.
- * use_mfma needs bf16 A and B; otherwise fp32 FMA accumulation in a fixed k order. */
+ * use_mfma needs bf16 A and B; otherwise fp32 FMA accumulation in a fixed k order.  bias (fp32 [N], may be NULL) is added to every row before epi. */
 int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t lda, int64_t a_bs, const void* B, int b_dt, int64_t sbn, int64_t sbk,
                 int64_t b_bs, void* C, int c_dt, int64_t ldc, int64_t c_bs, const int* grp_offs, const int* a_rows, int a_div, const int* c_rows,
-                const float* row_scale, int epi, int use_mfma, void* stream);
+                const float* row_scale, int epi, int use_mfma, const float* bias, void* stream);
 /* Causal attention with two-part keys over ragged batches: sequence s has n_new[s] query rows starting at row q_row0[s], `past[s]` earlier keys;
  * key j of it is K1 row k1_row0[s] + j (head stride k1_hs, D1 wide), K2 row k2_row0[s] + j (shared by heads, D2 wide), value row v_row0[s] + j.
  * Q fp32 [.., H, D1 + D2]; K1 / K2 / V / O of dtype dt.  A tile covers 32 / hm tokens x hm heads (hm > 1 needs k1_hs == v_hs == 0); the MFMA path (bf16,
  * D1 + D2 <= 320, DV <= 256) 128 / hm tokens, and with splits > 1 deals a tile's keys to that many workgroups whose partial results meet in ws
- * (n_seq * head tiles * token tiles * splits * 128 * (2 + DV rounded up to 32 / 64 / 128 / 256) floats). */
+ * (n_seq * head tiles * token tiles * splits * 128 * (2 + DV rounded up to 32 / 64 / 128 / 256) floats).
+ * Grouped queries: head h reads key / value head h / kv_rep (strides k1_hs / v_hs per key / value head; hm may then divide kv_rep).  window > 0: the query
+ * at position i sees key j <= i only if i - j < window or j < keep_first (a sliding window that keeps the first tokens); window 0: every j <= i. */
 int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, int D2, int DV, const float* Q, int64_t ldq, int q_hs, const void* K1, int64_t ldk1,
                       int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
                       const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
-                      int use_mfma, int splits, float* ws, int64_t ws_floats, void* stream);
+                      int use_mfma, int splits, float* ws, int64_t ws_floats, int kv_rep, int window, int keep_first, void* stream);
+
+/* ---- parallel-sublayer hybrid decoders in ragged batches (csrc/seqrec.hip) ---- */
+/* v = x + y1[t] + sum_{p < parts} y2[t * parts + p] (fp32 rows; y1 / y2 of dtype y*_dt, may be NULL); x_out (may be NULL or x) <- v.  For each weight
+ * w_a / w_b (fp32 [width], may be NULL): out[t, i] = v[i] / sqrt(mean of v^2 over i's group + eps) * w[i], the row cut into `groups` equal consecutive groups;
+ * written to out_* (dtype out_*_dt, may be NULL) and to out_*32 (fp32, may be NULL).  width <= 8192. */
+int mi355_group_rmsnorm_sum(int64_t tokens, int width, const float* x, const void* y1, int y1_dt, int64_t ldy1, const void* y2, int y2_dt, int64_t ldy2,
+                            int parts, float* x_out, int groups, float eps, const float* w_a, void* out_a, int out_a_dt, float* out_a32, const float* w_b,
+                            void* out_b, int out_b_dt, float* out_b32, void* stream);
+/* Causal convolution over time on every channel of ragged rows: y[t, c] = (residual ? x[t, c] : 0) + act(sum_j w[c, j] * in(t - taps + 1 + j, c)), w fp32
+ * [C, taps] (the last column weighs the current token); inputs before the step's first row come from state[slot[s]] (fp32 [slots, taps - 1, C], the inputs
+ * of the sequence's last taps - 1 tokens, zeros before its start), which afterwards holds the step's last inputs.  row_seq[t] = index of t's sequence
+ * in the step; act 0 none, 1 silu; taps <= 16. */
+int mi355_ragged_conv(int64_t tokens, int n_seq, int C, int taps, const void* x, int x_dt, int64_t ldx, const float* w, const int* row_seq, const int* seq_off,
+                      const int* slot, float* state, int act, int residual, void* y, int y_dt, int64_t ldy, void* stream);
+/* Query / key / value rows of grouped-query attention: src[t] = [H x d | G x d | G x dv] (+ bias fp32, may be NULL); query and key heads get an RMS norm over d
+ * (weights qw / kw fp32 [d], NULL: none) and a rotation of their first `dims` entries (layout as mi355_rope_heads); query head h times qscale[h] (may be NULL)
+ * goes to q_out fp32 [t, h * d]; key and value heads go to cache row dst_row[t] = [G x d | G x dv] of dtype c_dt. */
+int mi355_qkv_rows_append(int64_t tokens, int H, int G, int d, int dv, const void* src, int src_dt, int64_t ld_src, const float* bias, const float* qw,
+                          const float* kw, float eps, const float* qscale, int dims, int layout, const float* freq, const int* pos, const int* dst_row,
+                          float* q_out, int64_t ldq, void* cache, int c_dt, int64_t ldc, void* stream);
+/* Gated delta rule over the rows [seq_off[s], seq_off[s+1]) of each sequence, state[slot[s]] (fp32 [H, dk, dv]) read and written.  q / k rows [G * dk] (raw:
+ * made unit vectors here, x / sqrt(sum x^2 + 1e-6), q also times qscale), v rows [H * dv]; value head h uses query / key head h / (H / G);
+ * beta = sigmoid(b[t, h]), g = exp(-exp(A_log[h]) * softplus(a[t, h] + dt_bias[h])).  Per token: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
+ * o fp32 [tokens, H * dv].  dk <= 256. */
+int mi355_delta_rule_ragged(int n_seq, const int* seq_off, const int* slot, int H, int G, int dk, int dv, const void* q, const void* k, int qk_dt, int64_t ldq,
+                            int64_t ldk, const void* v, int v_dt, int64_t ldv, const void* b, const void* a, int ba_dt, int64_t ldb, int64_t lda,
+                            const float* A_log, const float* dt_bias, float qscale, float* state, float* o, void* stream);
+/* Gated feed-forward activation on rows [gate (F) | up (F)] -> [F].  kind 0: gelu_tanh(gate) * up.  kind 1: g = min(gate, limit), u = clamp(up, -limit, limit),
+ * g * sigmoid(1.702 g) * (u + 1). */
+int mi355_glu_rows(int64_t rows, int F, const void* in, int in_dt, int64_t ld_in, int kind, float limit, void* out, int out_dt, int64_t ld_out, void* stream);
 
 #ifdef __cplusplus
 }

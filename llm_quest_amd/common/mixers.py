@@ -42,8 +42,9 @@ class SeqStep:
         self.host_seq_off = seq_off
         T, n = self.T, self.n_seq
         row0 = [s * cap for s in slots]
-        # rows of the descriptor block: tokens | previous token | position | cache row | per-sequence arrays | 0 .. T-1; one host-to-device copy for all
-        buf = np.empty(5 * T + 5 * n + 1, dtype=np.int32)
+        # rows of the descriptor block: tokens | previous token | position | cache row | per-sequence arrays | 0 .. T-1 | sequence of a row; one
+        # host-to-device copy for all
+        buf = np.empty(6 * T + 5 * n + 1, dtype=np.int32)
         tok, prev, pos, dst = buf[0:T], buf[T : 2 * T], buf[2 * T : 3 * T], buf[3 * T : 4 * T]
         for i, (slot, new) in enumerate(entries):
             a, b = seq_off[i], seq_off[i + 1]
@@ -57,13 +58,14 @@ class SeqStep:
             buf[at : at + len(arr)] = arr
             at += len(arr)
         buf[at : at + T] = np.arange(T, dtype=np.int32)
+        buf[at + T : at + 2 * T] = np.repeat(np.arange(n, dtype=np.int32), n_new)
         buf = torch.from_numpy(buf).to(device, non_blocking=False)
-        cuts = [T, T, T, T, n + 1, n, n, n, n, T]
+        cuts = [T, T, T, T, n + 1, n, n, n, n, T, T]
         parts, at = [], 0
         for c in cuts:
             parts.append(buf[at : at + c])
             at += c
-        (self.tok, self.prev, self.pos, self.dst_row, self.seq_off, self.slots, self.past, self.n_new, self.cache_row0, self.local_row) = parts
+        (self.tok, self.prev, self.pos, self.dst_row, self.seq_off, self.slots, self.past, self.n_new, self.cache_row0, self.local_row, self.row_seq) = parts
         self.q_row0 = self.seq_off[:n]
         self.local = {}  # layer -> this step's latent rows [T, rank + rot] (prompts: the expanded form reads them instead of the cache)
 
@@ -219,4 +221,214 @@ class GroupedSigmoidMoE(_Frozen):
         S.bgemm(h, self.w_up, act, T * top, self.ff, self.width, batch=E, sbn=self.width, b_bs=self.ff * self.width, grp_offs=offs, a_rows=perm, a_div=top, epi=1)
         out = torch.empty((T * top, self.width), dtype=F32, device=h.device)
         S.bgemm(act, self.w_down, out, T * top, self.width, self.ff, batch=E, sbn=self.ff, b_bs=self.width * self.ff, grp_offs=offs, c_rows=perm, row_scale=wts.view(-1))
+        return out
+
+
+# ----------------------------------------------------------------------------------------------- mechanisms of parallel-sublayer hybrid decoders
+def _largest_pow2_divisor(n, cap=32):
+    p = 1
+    while p * 2 <= cap and n % (p * 2) == 0:
+        p *= 2
+    return p
+
+
+class ShortConvInput(_Frozen):
+    """h <- h + conv(h): a causal convolution over time on every channel (``taps`` wide, no bias), added to its input.  The last ``taps - 1`` inputs of
+    every sequence are carried as the state ``name`` of the layer."""
+
+    def __init__(self, channels, taps, layer_idx, name="canon"):
+        super().__init__()
+        self.channels, self.taps, self.layer_idx, self.name = channels, taps, layer_idx, name
+        self.weight = self._param(channels, taps)
+        self._ready = None
+
+    def state_spec(self):
+        return {self.name: (self.taps - 1, self.channels)} if self.taps > 1 else {}
+
+    def prepare(self, device):
+        if self._ready != device:
+            self.weight32 = _f32(self.weight)
+            self._ready = device
+
+    @torch.no_grad()
+    def step(self, h32, st, out_dtype):
+        """h32: fp32 rows -> h + conv(h) in ``out_dtype`` (one rounding, after the sum)."""
+        self.prepare(h32.device)
+        state = st.cache.state(self.layer_idx, self.name) if self.taps > 1 else None
+        return S.ragged_conv(h32, self.weight32, state, st.row_seq, st.seq_off, st.slots, act=False, residual=True, out_dtype=out_dtype)
+
+
+class Retention(_Frozen):
+    """Linear attention with ONE fixed decay per head and no softmax or denominator: S <- decay_h S + k v^T, o = S^T q, the state carried in fp32.
+    Rotary positions on q and k in the rotate-half layout (entry i pairs with i + rot_dims / 2); k is scaled by dim^-1/2 after the rotation; every head's
+    output is divided by its root mean square, gated by silu of a projection, and projected out."""
+
+    def __init__(self, width, heads, dim, vdim, decay, rot_dims, rot_base, eps, layer_idx):
+        super().__init__()
+        if len(decay) != heads:
+            raise ValueError(f"Retention: {len(decay)} decays for {heads} heads")
+        if rot_dims % 2 or rot_dims > dim:
+            raise ValueError("Retention: the rotated entries are an even number <= dim")
+        self.width, self.heads, self.dim, self.vdim, self.decay, self.rot_dims, self.rot_base, self.eps, self.layer_idx = width, heads, dim, vdim, [float(d) for d in decay], rot_dims, float(rot_base), float(eps), layer_idx
+        self.w_in = self._param(2 * heads * dim + 2 * heads * vdim, width)  # [q | k | v | gate] rows -> one product
+        self.w_o = self._param(width, heads * vdim)
+        self._ready = None
+
+    def cache_spec(self):
+        return {"rows": None, "states": {"S": (self.heads, self.dim, self.vdim)}}
+
+    def prepare(self, device):
+        if self._ready != device:
+            self.decay32 = torch.tensor(self.decay, dtype=torch.float64).to(F32).to(device)
+            self.freq = S.rope_frequencies(self.rot_dims, self.rot_base, device) if self.rot_dims else None
+            self.ones = torch.ones(self.vdim, dtype=F32, device=device)
+            self._ready = device
+
+    @torch.no_grad()
+    def step(self, h, st):
+        self.prepare(h.device)
+        H, dk, dv = self.heads, self.dim, self.vdim
+        proj = S.linear(h, self.w_in, out_dtype=F32)
+        a, b, c = H * dk, 2 * H * dk, 2 * H * dk + H * dv
+        qk = torch.empty((h.shape[0], b), dtype=F32, device=h.device)
+        S.rope_heads(proj, 2 * H, dk, dk, 0, qk, dk, 0, 0, self.rot_dims, self.freq, st.pos, layout=1)  # q and k heads side by side: 2 H heads of dim
+        o = S.gla(qk[:, :a], qk[:, a:b], proj[:, b:c], None, None, 1.0, 1.0, st.seq_off, st.slots, st.cache.state(self.layer_idx, "S"), H, dk, dv,
+                  head_decay=self.decay32, kscale=dk ** -0.5)
+        mix = S.gated_headnorm(o, self.ones, proj[:, c:], H, dv, self.eps, st.act_dtype)
+        return S.linear(mix, self.w_o)
+
+
+class SlidingWindowAttention(_Frozen):
+    """Grouped-query softmax attention with biases on the four projections, an RMS norm (one weight for all heads) on every query and key head before
+    an interleaved rotary embedding of the first ``rot_dims`` entries, score = q.k * scale * temp[h], and a causal sliding window that also keeps the
+    first tokens: position i sees j <= i if i - j < window or j < keep_first (window 0: all of them).  Keys and values are cached token-major,
+    [kv_heads x dim | kv_heads x vdim] per row."""
+
+    def __init__(self, width, heads, kv_heads, dim, vdim, scale, window, keep_first, rot_dims, rot_base, eps, layer_idx, qk_norm=True, bias=True, temp=True):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("SlidingWindowAttention: heads must be a multiple of kv_heads")
+        if rot_dims % 2 or rot_dims > dim:
+            raise ValueError("SlidingWindowAttention: the rotated entries are an even number <= dim")
+        self.width, self.heads, self.kv_heads, self.dim, self.vdim, self.scale, self.window, self.keep_first = width, heads, kv_heads, dim, vdim, float(scale), int(window), int(keep_first)
+        self.rot_dims, self.rot_base, self.eps, self.layer_idx = rot_dims, float(rot_base), float(eps), layer_idx
+        n = (heads + kv_heads) * dim + kv_heads * vdim
+        self.w_qkv = self._param(n, width)
+        self.b_qkv = self._param(n) if bias else None
+        self.q_norm = self._param(dim) if qk_norm else None
+        self.k_norm = self._param(dim) if qk_norm else None
+        self.temp = self._param(heads) if temp else None
+        self.w_o = self._param(width, heads * vdim)
+        self.b_o = self._param(width) if bias else None
+        self._ready = None
+
+    def cache_spec(self):
+        return {"rows": self.kv_heads * (self.dim + self.vdim), "states": {}}
+
+    def prepare(self, device):
+        if self._ready != device:
+            self.b_qkv32, self.q_norm32, self.k_norm32, self.b_o32 = _f32(self.b_qkv), _f32(self.q_norm), _f32(self.k_norm), _f32(self.b_o)
+            t = _f32(self.temp) if self.temp is not None else torch.ones(self.heads, dtype=F32, device=device)
+            self.qscale = (t * self.scale).contiguous()  # the score's two factors, folded onto the query
+            self.freq = S.rope_frequencies(self.rot_dims, self.rot_base, device) if self.rot_dims else None
+            self._ready = device
+
+    @torch.no_grad()
+    def step(self, h, st):
+        self.prepare(h.device)
+        H, G, d, dv = self.heads, self.kv_heads, self.dim, self.vdim
+        cache2d = st.cache.rows2d(self.layer_idx)
+        proj = S.linear(h, self.w_qkv, out_dtype=F32)
+        q = S.qkv_rows_append(proj, H, G, d, dv, self.b_qkv32, self.q_norm32, self.k_norm32, self.eps, self.qscale, self.rot_dims, 0, self.freq, st.pos, st.dst_row, cache2d)
+        ctx = torch.empty((h.shape[0], H * dv), dtype=st.act_dtype, device=h.device)
+        hm = _largest_pow2_divisor(H // G)
+        S.latent_attn(q, cache2d, None, cache2d[:, G * d :], ctx, H, hm, d, 0, dv, d, d, dv, dv, (st.q_row0, st.n_new, st.past, st.cache_row0, st.cache_row0, st.cache_row0),
+                      st.max_new, 1.0, max_keys=st.max_keys, kv_rep=H // G, window=self.window, keep_first=self.keep_first)
+        return S.linear(ctx, self.w_o, bias=self.b_o32)
+
+
+class GatedDeltaRule(_Frozen):
+    """Gated delta rule with a matrix state per value head, carried in fp32.  q / k (``kv_heads`` x dim) and v (``heads`` x vdim) pass a short causal
+    convolution per channel and silu; q and k become unit vectors per head (q also times dim^-1/2); beta = sigmoid(W_b h); one decay per head,
+    g = exp(-exp(A_log) softplus(W_a h + dt_bias)); S <- g S, u = beta (v - S^T k), S <- S + k u^T, o = S^T q.  Every head's output is RMS-normed with
+    one weight [vdim], gated by silu of a projection, and projected out."""
+
+    def __init__(self, width, heads, kv_heads, dim, vdim, conv_taps, eps, layer_idx):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("GatedDeltaRule: heads must be a multiple of kv_heads")
+        self.width, self.heads, self.kv_heads, self.dim, self.vdim, self.conv_taps, self.eps, self.layer_idx = width, heads, kv_heads, dim, vdim, conv_taps, float(eps), layer_idx
+        self.channels = 2 * kv_heads * dim + heads * vdim
+        self.w_in = self._param(self.channels + heads * vdim + 2 * heads, width)  # [q | k | v | gate | b | a] rows -> one product
+        self.conv = self._param(self.channels, conv_taps)
+        self.A_log, self.dt_bias = self._param(heads), self._param(heads)
+        self.norm = self._param(vdim)
+        self.w_o = self._param(width, heads * vdim)
+        self._ready = None
+
+    def cache_spec(self):
+        states = {"S": (self.heads, self.dim, self.vdim)}
+        if self.conv_taps > 1:
+            states["conv"] = (self.conv_taps - 1, self.channels)
+        return {"rows": None, "states": states}
+
+    def prepare(self, device):
+        if self._ready != device:
+            self.conv32, self.A_log32, self.dt_bias32, self.norm32 = _f32(self.conv), _f32(self.A_log), _f32(self.dt_bias), _f32(self.norm)
+            self._ready = device
+
+    @torch.no_grad()
+    def step(self, h, st):
+        self.prepare(h.device)
+        H, G, dk, dv, C = self.heads, self.kv_heads, self.dim, self.vdim, self.channels
+        proj = S.linear(h, self.w_in, out_dtype=F32)
+        state = st.cache.state(self.layer_idx, "conv") if self.conv_taps > 1 else None
+        qkv = S.ragged_conv(proj[:, :C], self.conv32, state, st.row_seq, st.seq_off, st.slots, act=True, residual=False, out_dtype=F32)
+        a, b = G * dk, 2 * G * dk
+        gate0 = C + H * dv
+        o = S.delta_rule(qkv[:, :a], qkv[:, a:b], qkv[:, b:], proj[:, gate0 : gate0 + H], proj[:, gate0 + H :], self.A_log32, self.dt_bias32, dk ** -0.5, st.seq_off, st.slots,
+                         st.cache.state(self.layer_idx, "S"), H, G, dk, dv)
+        mix = S.gated_headnorm(o, self.norm32, proj[:, C:gate0], H, dv, self.eps, st.act_dtype)
+        return S.linear(mix, self.w_o)
+
+
+class GatedMLP(_Frozen):
+    """Dense gated feed-forward: down(act(gate x) * (up x)), act = the tanh form of GELU; gate and up are one product."""
+
+    def __init__(self, width, ff):
+        super().__init__()
+        self.width, self.ff = width, ff
+        self.w_gate_up = self._param(2 * ff, width)
+        self.w_down = self._param(width, ff)
+        self.top = 1
+
+    @torch.no_grad()
+    def step(self, h32, h):
+        return S.linear(S.glu_rows(S.linear(h, self.w_gate_up), S.GLU_GELU_TANH), self.w_down)
+
+
+class SoftmaxTopkMoE(_Frozen):
+    """``experts`` gated feed-forward experts without biases, ``top`` per token.  Router: fp32 logits, softmax over ALL experts, the ``top`` largest scores
+    win and ARE the weights (not renormalised).  Expert: g = min(gate x, limit), u = clamp(up x, -limit, limit), down(g sigmoid(1.702 g) (u + 1)).
+    Returns the weighted outputs as ``top`` fp32 rows per token; the sum is taken by the residual kernel that follows."""
+
+    def __init__(self, width, ff, experts, top, limit):
+        super().__init__()
+        self.width, self.ff, self.experts, self.top, self.limit = width, ff, experts, top, float(limit)
+        self.w_router = self._param(experts, width)
+        self.w_gate_up = self._param(experts, 2 * ff, width)
+        self.w_down = self._param(experts, width, ff)
+
+    @torch.no_grad()
+    def step(self, h32, h):
+        """h32: the normed fp32 rows (the router reads them), h: the same rows in the activation dtype -> fp32 [T * top, width]."""
+        T, E, top, ff = h.shape[0], self.experts, self.top, self.ff
+        logits = S.router_logits(h32, self.w_router)
+        ids, wts = S.moe_route(logits, None, top, 1, 1, 1.0, softmax=True)
+        offs, perm = S.moe_dispatch(ids.view(-1), E)
+        gu = torch.empty((T * top, 2 * ff), dtype=h.dtype, device=h.device)
+        S.bgemm(h, self.w_gate_up, gu, T * top, 2 * ff, self.width, batch=E, sbn=self.width, b_bs=2 * ff * self.width, grp_offs=offs, a_rows=perm, a_div=top)
+        act = S.glu_rows(gu, S.GLU_CLAMPED_SWISH, self.limit)
+        out = torch.empty((T * top, self.width), dtype=F32, device=h.device)
+        S.bgemm(act, self.w_down, out, T * top, self.width, ff, batch=E, sbn=ff, b_bs=self.width * ff, grp_offs=offs, c_rows=perm, row_scale=wts.view(-1))
         return out

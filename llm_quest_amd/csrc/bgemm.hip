@@ -30,6 +30,7 @@ struct BgemmArgs {
     int a_div;
     const int* c_rows;       // or null: sorted row r writes C row c_rows[r]
     const float* row_scale;  // or null: C row (after c_rows) is multiplied by row_scale[that row]
+    const float* bias;       // or null: bias[n] is added to column n before the epilogue
     int epi;                 // 0 none, 1 relu(x)^2
     int a_dt, b_dt, c_dt;
 };
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(256) void bgemm_fma_kernel(BgemmArgs p) {
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
             if (n >= p.N) continue;
-            float v = acc[i][j];
+            float v = acc[i][j] + (p.bias ? p.bias[n] : 0.f);
             if (p.epi == 1) v = v > 0.f ? v * v : 0.f;
             v *= sc;
             if (p.c_dt == MI355_DT_F32) ((float*)p.C)[cb + n] = v;
@@ -195,7 +196,7 @@ __global__ __launch_bounds__(256) void bgemm_mfma_kernel(BgemmArgs p) {
             const int r = row0 + m;
             const int64_t crow = p.c_rows ? p.c_rows[r] : r;
             const float sc = p.row_scale ? p.row_scale[crow] : 1.0f;
-            float v = acc[4 * g + i];
+            float v = acc[4 * g + i] + (p.bias ? p.bias[n] : 0.f);
             if (p.epi == 1) v = v > 0.f ? v * v : 0.f;
             v *= sc;
             const int64_t ci = (int64_t)b * p.c_bs + crow * p.ldc + n;
@@ -310,7 +311,7 @@ __global__ __launch_bounds__(256) void bgemm_mfma128_kernel(BgemmArgs p) {
                 for (int bj = 0; bj < 2; ++bj) {
                     const int n = n0 + wn + 32 * bj + ln;
                     if (n >= p.N) continue;
-                    float v = acc[bi][bj][4 * g + i];
+                    float v = acc[bi][bj][4 * g + i] + (p.bias ? p.bias[n] : 0.f);
                     if (p.epi == 1) v = v > 0.f ? v * v : 0.f;
                     v *= sc;
                     if (p.c_dt == MI355_DT_F32) ((float*)p.C)[cb + n] = v;
@@ -321,7 +322,7 @@ __global__ __launch_bounds__(256) void bgemm_mfma128_kernel(BgemmArgs p) {
 
 extern "C" int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t lda, int64_t a_bs, const void* B, int b_dt, int64_t sbn, int64_t sbk,
                            int64_t b_bs, void* C, int c_dt, int64_t ldc, int64_t c_bs, const int* grp_offs, const int* a_rows, int a_div, const int* c_rows,
-                           const float* row_scale, int epi, int use_mfma, void* stream) {
+                           const float* row_scale, int epi, int use_mfma, const float* bias, void* stream) {
     MI355_REQUIRE(batch > 0 && batch <= 65535 && M > 0 && N > 0 && K > 0 && A && B && C, "bgemm: bad arguments");
     MI355_REQUIRE((a_dt == MI355_DT_BF16 || a_dt == MI355_DT_F32) && (b_dt == MI355_DT_BF16 || b_dt == MI355_DT_F32) && (c_dt == MI355_DT_BF16 || c_dt == MI355_DT_F32),
                   "bgemm: bad dtype");
@@ -334,6 +335,7 @@ extern "C" int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_
     p.lda = lda, p.a_bs = a_bs, p.sbn = sbn, p.sbk = sbk, p.b_bs = b_bs, p.ldc = ldc, p.c_bs = c_bs;
     p.M = M, p.N = N, p.K = K;
     p.grp_offs = grp_offs, p.a_rows = a_rows, p.a_div = a_rows ? a_div : 1, p.c_rows = c_rows, p.row_scale = row_scale;
+    p.bias = bias;
     p.epi = epi, p.a_dt = a_dt, p.b_dt = b_dt, p.c_dt = c_dt;
     if (use_mfma && sbk == 1 && N >= 128 && K >= 64) {  // the large tile: weights stored [out, in], enough columns to fill it
         const int64_t my128 = ((int64_t)M + TM - 1) / TM;

@@ -5,6 +5,8 @@
 //     K1 = V = the cached latent rows themselves (head stride 0), K2 = the cached rotated part: the cache is read once for all heads.
 //
 // score(row, j) = scale * ( Q[row, :D1] . K1[j, head, :] + Q[row, D1:] . K2[j, :] ),  softmax over j <= past + token index, out = sum_j p V[j].
+// The same kernels serve grouped-query attention (kv_rep query heads per key / value head, D2 = 0) and a sliding window that keeps the first tokens
+// (window, keep_first): key steps that no row of a tile can see are skipped.
 // Scores, softmax statistics and the output accumulators are fp32.  A tile is `tm` tokens x `hm` heads = 32 query rows (hm > 1 only with shared
 // keys and values) against 64 keys at a time.
 //
@@ -26,7 +28,13 @@ struct LatAttnArgs {
     float scale;
     int splits;  // MFMA path: a tile's keys are dealt to `splits` workgroups; partial (max, sum, output) rows go to ws and latent_attn_combine_kernel joins them
     float* ws;   // per (sequence, head tile, token tile, split): 128 maxima | 128 sums | 128 x DVP unnormalised outputs
+    int kv_rep;  // query heads per key / value head (grouped queries): head h reads key / value head h / kv_rep
+    int window;  // > 0: a query at position i sees key j <= i only if i - j < window or j < keep_first (sliding window that keeps the first tokens)
+    int keep_first;
 };
+
+// key j for the query at position lim (lim < 0: a padding row that sees nothing)
+__device__ __forceinline__ bool key_visible(int j, int lim, int window, int keep_first) { return j <= lim && (window <= 0 || lim - j < window || j < keep_first); }
 
 __device__ __forceinline__ float lda_dt(const void* p, int dt, int64_t i) { return dt == MI355_DT_F32 ? ((const float*)p)[i] : bf2f(((const bf16_t*)p)[i]); }
 
@@ -64,7 +72,10 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
 #pragma unroll
         for (int i = 0; i < NC; ++i) o[r][i] = 0.f;
 
+    const int kvh = head0 / p.kv_rep;
+    const int win_lo = p.window > 0 ? past + tok0 - p.window + 1 : 0;  // keys below it are outside the window of every row of the tile
     for (int j0 = 0; j0 < n_keys; j0 += AN) {
+        if (j0 + AN <= win_lo && j0 >= p.keep_first) continue;  // block-uniform: no row sees a key of this step
         float acc[2][4] = {};
         for (int d0 = 0; d0 < DK; d0 += AC) {
             __syncthreads();
@@ -79,7 +90,7 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
                 const int e = tid + 256 * i, d = d0 + (e & 31), j = j0 + (e >> 5);
                 float v = 0.f;
                 if (j < n_keys && d < DK)
-                    v = d < p.D1 ? lda_dt(p.K1, p.dt, (k1r0 + j) * p.ldk1 + (int64_t)head0 * p.k1_hs + d) : lda_dt(p.K2, p.dt, (k2r0 + j) * p.ldk2 + (d - p.D1));
+                    v = d < p.D1 ? lda_dt(p.K1, p.dt, (k1r0 + j) * p.ldk1 + (int64_t)kvh * p.k1_hs + d) : lda_dt(p.K2, p.dt, (k2r0 + j) * p.ldk2 + (d - p.D1));
                 Ks[e >> 5][e & 31] = v;
             }
             __syncthreads();
@@ -101,7 +112,7 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int j = j0 + tx + 16 * i;
-                acc[a][i] = j <= lim[a] ? acc[a][i] * p.scale : -__builtin_huge_valf();
+                acc[a][i] = key_visible(j, lim[a], p.window, p.keep_first) ? acc[a][i] * p.scale : -__builtin_huge_valf();
                 mx = fmaxf(mx, acc[a][i]);
             }
 #pragma unroll
@@ -136,7 +147,7 @@ __global__ __launch_bounds__(256) void latent_attn_fma_kernel(LatAttnArgs p) {
 #pragma unroll
             for (int i = 0; i < NC; ++i) {
                 const int col = c + 64 * i;
-                vv[i] = col < p.DV ? lda_dt(p.V, p.dt, (vr0 + j0 + j) * p.ldv + (int64_t)head0 * p.v_hs + col) : 0.f;
+                vv[i] = col < p.DV ? lda_dt(p.V, p.dt, (vr0 + j0 + j) * p.ldv + (int64_t)kvh * p.v_hs + col) : 0.f;
             }
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
@@ -230,7 +241,10 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
     float m_run = NEG, l_run = 0.f;
     const float sc2 = p.scale * 1.4426950408889634f;
 
+    const int kvh = head0 / p.kv_rep;
+    const int win_lo = p.window > 0 ? past + tok0 - p.window + 1 : 0;
     for (int j0 = key_lo; j0 < n_keys; j0 += MKT) {
+        if (j0 + MKT <= win_lo && j0 >= p.keep_first) continue;  // block-uniform: no row sees a key of this step
         __syncthreads();
         // ---- key tile -> LDS
         for (int c = tid; c < MKT * DKS; c += 256) {
@@ -238,7 +252,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
             u32x4 val = {0u, 0u, 0u, 0u};
             if (j < n_keys) {
                 if (vec_ok && d0 + 8 <= p.D1) {
-                    val = *(const u32x4*)(K1 + (k1r0 + j) * p.ldk1 + (int64_t)head0 * p.k1_hs + d0);
+                    val = *(const u32x4*)(K1 + (k1r0 + j) * p.ldk1 + (int64_t)kvh * p.k1_hs + d0);
                 } else if (vec_ok && d0 >= p.D1 && d0 + 8 <= DK) {
                     val = *(const u32x4*)(K2 + (k2r0 + j) * p.ldk2 + (d0 - p.D1));
                 } else {
@@ -246,7 +260,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
                         const int d = d0 + i;
-                        e[i] = d < p.D1 ? K1[(k1r0 + j) * p.ldk1 + (int64_t)head0 * p.k1_hs + d] : (d < DK ? K2[(k2r0 + j) * p.ldk2 + (d - p.D1)] : (bf16_t)0);
+                        e[i] = d < p.D1 ? K1[(k1r0 + j) * p.ldk1 + (int64_t)kvh * p.k1_hs + d] : (d < DK ? K2[(k2r0 + j) * p.ldk2 + (d - p.D1)] : (bf16_t)0);
                     }
                     val = u32x4{(unsigned)e[0] | ((unsigned)e[1] << 16), (unsigned)e[2] | ((unsigned)e[3] << 16), (unsigned)e[4] | ((unsigned)e[5] << 16),
                                 (unsigned)e[6] | ((unsigned)e[7] << 16)};
@@ -261,12 +275,12 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
             const int key = c % MKT, v0 = (c / MKT) * 8, j = j0 + key;
             bf16_t e[8];
             if (j < n_keys && vec_ok && v0 + 8 <= p.DV) {
-                const u32x4 val = *(const u32x4*)(V + (vr0 + j) * p.ldv + (int64_t)head0 * p.v_hs + v0);
+                const u32x4 val = *(const u32x4*)(V + (vr0 + j) * p.ldv + (int64_t)kvh * p.v_hs + v0);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) e[2 * i] = (bf16_t)(val[i] & 0xffffu), e[2 * i + 1] = (bf16_t)(val[i] >> 16);
             } else {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) e[i] = (j < n_keys && v0 + i < p.DV) ? V[(vr0 + j) * p.ldv + (int64_t)head0 * p.v_hs + v0 + i] : (bf16_t)0;
+                for (int i = 0; i < 8; ++i) e[i] = (j < n_keys && v0 + i < p.DV) ? V[(vr0 + j) * p.ldv + (int64_t)kvh * p.v_hs + v0 + i] : (bf16_t)0;
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i) Vt[(v0 + i) * VLD + key] = e[i];
@@ -292,7 +306,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatAttnArgs p, in
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int j = j0 + kb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
-                const float v = (j <= lim && j < n_keys) ? sacc[kb][r] * sc2 : NEG;
+                const float v = (key_visible(j, lim, p.window, p.keep_first) && j < n_keys) ? sacc[kb][r] * sc2 : NEG;
                 sacc[kb][r] = v;
                 mx = fmaxf(mx, v);
             }
@@ -396,14 +410,16 @@ static int launch_mfma(const LatAttnArgs& p, dim3 grid, int vec_ok, hipStream_t 
 extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, int D2, int DV, const float* Q, int64_t ldq, int q_hs, const void* K1, int64_t ldk1,
                                  int k1_hs, const void* K2, int64_t ldk2, const void* V, int64_t ldv, int v_hs, void* O, int64_t ldo, int o_hs, int dt,
                                  const int* q_row0, const int* n_new, const int* past, const int* k1_row0, const int* k2_row0, const int* v_row0, float scale,
-                                 int use_mfma, int splits, float* ws, int64_t ws_floats, void* stream) {
+                                 int use_mfma, int splits, float* ws, int64_t ws_floats, int kv_rep, int window, int keep_first, void* stream) {
     MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && max_new > 0 && H > 0 && D1 > 0 && D2 >= 0 && DV > 0 && DV <= 512 && Q && K1 && V && O && (D2 == 0 || K2),
                   "latent_attn: bad arguments (value width <= 512)");
     MI355_REQUIRE(dt == MI355_DT_BF16 || dt == MI355_DT_F32, "latent_attn: bad dtype");
-    MI355_REQUIRE(hm >= 1 && hm <= AM && AM % hm == 0 && (hm == 1 || (k1_hs == 0 && v_hs == 0)), "latent_attn: several heads per tile (a power of two <= 32) need shared keys and values (head stride 0)");
+    MI355_REQUIRE(kv_rep >= 1 && H % kv_rep == 0 && window >= 0 && keep_first >= 0, "latent_attn: bad head grouping or window");
+    MI355_REQUIRE(hm >= 1 && hm <= AM && AM % hm == 0 && (hm == 1 || (k1_hs == 0 && v_hs == 0) || kv_rep % hm == 0),
+                  "latent_attn: several heads per tile (a power of two <= 32) need shared keys and values (head stride 0, or one key / value head for the tile's heads)");
     MI355_REQUIRE(!use_mfma || dt == MI355_DT_BF16, "latent_attn: the MFMA path takes bf16 keys and values");
     MI355_REQUIRE(q_row0 && n_new && past && k1_row0 && k2_row0 && v_row0, "latent_attn: sequence descriptors missing");
-    MI355_REQUIRE(ldq >= (int64_t)(H - 1) * q_hs + D1 + D2 && ldo >= (int64_t)(H - 1) * o_hs + DV && ldk1 >= (int64_t)(H - 1) * k1_hs + D1 && ldv >= (int64_t)(H - 1) * v_hs + DV &&
+    MI355_REQUIRE(ldq >= (int64_t)(H - 1) * q_hs + D1 + D2 && ldo >= (int64_t)(H - 1) * o_hs + DV && ldk1 >= (int64_t)((H - 1) / kv_rep) * k1_hs + D1 && ldv >= (int64_t)((H - 1) / kv_rep) * v_hs + DV &&
                       (D2 == 0 || ldk2 >= D2),
                   "latent_attn: rows too short");
     LatAttnArgs p;
@@ -413,6 +429,7 @@ extern "C" int mi355_latent_attn(int n_seq, int max_new, int H, int hm, int D1, 
     p.D1 = D1, p.D2 = D2, p.DV = DV, p.H = H, p.hm = hm, p.dt = dt;
     p.q_row0 = q_row0, p.n_new = n_new, p.past = past, p.k1_row0 = k1_row0, p.k2_row0 = k2_row0, p.v_row0 = v_row0;
     p.scale = scale;
+    p.kv_rep = kv_rep, p.window = window, p.keep_first = keep_first;
     p.splits = 1, p.ws = nullptr;
     const bool mfma = use_mfma && D1 + D2 <= 320 && DV <= 256;  // what the MFMA kernel keeps in registers; larger heads take the FMA path
     const int tm = (mfma ? MQ : AM) / hm;

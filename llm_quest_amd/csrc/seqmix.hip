@@ -277,10 +277,11 @@ extern "C" int mi355_latent_kv_append(int64_t tokens, int rank, int rot, const v
     return 0;
 }
 
-// Copy n entries per head from src to dst (fp32) and turn the pairs of [rot_start, rot_start + dims):
+// Copy n entries per head from src to dst (fp32) and turn the pairs of [rot_start, rot_start + dims) -- layout 0: neighbours (2i, 2i+1); layout 1: the
+// two halves of the range, (i, i + dims/2):
 // dst[t, h * dst_hs + dst_off + i] = src[t, h * src_hs + src_off + i]
 __global__ __launch_bounds__(256) void rope_heads_kernel(int64_t T, int H, int n, const void* __restrict__ src, int src_dt, int64_t lds_, int src_hs, int src_off,
-                                                         float* __restrict__ dst, int64_t ldd, int dst_hs, int dst_off, int rot_start, int dims,
+                                                         float* __restrict__ dst, int64_t ldd, int dst_hs, int dst_off, int rot_start, int dims, int layout,
                                                          const float* __restrict__ freq, const int* __restrict__ pos) {
     const int lane = threadIdx.x & 63;
     const int64_t items = T * H;
@@ -293,22 +294,23 @@ __global__ __launch_bounds__(256) void rope_heads_kernel(int64_t T, int H, int n
         for (int i = lane; i < n; i += 64)
             if (i < rot_start || i >= rot_start + dims) dst[dof + i] = ld_dt(src, src_dt, so + i);
         for (int i = lane; i < dims / 2; i += 64) {
-            const float u = ld_dt(src, src_dt, so + rot_start + 2 * i), v = ld_dt(src, src_dt, so + rot_start + 2 * i + 1);
+            const int a = rot_start + (layout ? i : 2 * i), b = rot_start + (layout ? i + dims / 2 : 2 * i + 1);
+            const float u = ld_dt(src, src_dt, so + a), v = ld_dt(src, src_dt, so + b);
             float ou, ov;
             turn_pair(u, v, p * freq[i], ou, ov);
-            dst[dof + rot_start + 2 * i] = ou;
-            dst[dof + rot_start + 2 * i + 1] = ov;
+            dst[dof + a] = ou;
+            dst[dof + b] = ov;
         }
     }
 }
 
 extern "C" int mi355_rope_heads(int64_t tokens, int H, int n, const void* src, int src_dt, int64_t ld_src, int src_hs, int src_off, float* dst, int64_t ld_dst,
-                                int dst_hs, int dst_off, int rot_start, int dims, const float* freq, const int* pos, void* stream) {
-    MI355_REQUIRE(tokens > 0 && H > 0 && n > 0 && src && dst && pos && dt_ok(src_dt), "rope_heads: bad arguments");
+                                int dst_hs, int dst_off, int rot_start, int dims, int layout, const float* freq, const int* pos, void* stream) {
+    MI355_REQUIRE(tokens > 0 && H > 0 && n > 0 && src && dst && pos && dt_ok(src_dt) && (layout == 0 || layout == 1), "rope_heads: bad arguments");
     MI355_REQUIRE(rot_start >= 0 && dims >= 0 && dims % 2 == 0 && rot_start + dims <= n && (dims == 0 || freq), "rope_heads: the rotated range must lie inside the head");
     MI355_REQUIRE(src_off >= 0 && dst_off >= 0 && ld_src >= (int64_t)(H - 1) * src_hs + src_off + n && ld_dst >= (int64_t)(H - 1) * dst_hs + dst_off + n, "rope_heads: rows too short");
     rope_heads_kernel<<<rows_grid(tokens * H, 4), 256, 0, ST(stream)>>>(tokens, H, n, src, src_dt, ld_src, src_hs, src_off, dst, ld_dst, dst_hs, dst_off, rot_start, dims,
-                                                                      freq, pos);
+                                                                      layout, freq, pos);
     MI355_LAUNCH_CHECK("rope_heads");
     return 0;
 }
@@ -345,7 +347,8 @@ extern "C" int mi355_gated_headnorm(int64_t tokens, int H, int D, const float* o
 
 // ------------------------------------------------------------------------------------------- gated linear attention
 // Per head a state S [dk, dv] (fp32, carried per sequence slot):  S <- diag(a_t) S + k_t v_t^T,  o_t = S^T (q_t * qscale),
-// a_t = sigmoid(z_t + zbias)^(inv_tau) = exp(inv_tau * logsigmoid(.)) in fp32.
+// a_t = sigmoid(z_t + zbias)^(inv_tau) = exp(inv_tau * logsigmoid(.)) in fp32 -- or, with head_decay, the constant head_decay[h] for every key channel
+// of head h (retention: z / zbias are then unused).  k_t is multiplied by kscale.
 // Block: 64 value columns x RC row chunks of GLA_R key channels; a thread keeps GLA_R state entries of one column in registers.
 // Tokens go through in groups of GLA_TB: the group's q / k / decay rows are staged in LDS once, partial outputs of the row chunks meet in LDS.
 #define GLA_R 16
@@ -354,7 +357,8 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 
 __global__ void gla_kernel(const int* __restrict__ seq_off, const int* __restrict__ slot, int H, int dk, int dv, const void* __restrict__ q, const void* __restrict__ k,
                            const void* __restrict__ v, const void* __restrict__ z, int dt, int z_dt, int64_t ldq, int64_t ldk, int64_t ldv_, int64_t ldz,
-                           const float* __restrict__ zbias, float inv_tau, float qscale, float* __restrict__ state, float* __restrict__ o) {
+                           const float* __restrict__ zbias, float inv_tau, float qscale, const float* __restrict__ head_decay, float kscale,
+                           float* __restrict__ state, float* __restrict__ o) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int RC = blockDim.x >> 6;
     float* sq = smem;                       // [TB][dk]
@@ -386,7 +390,7 @@ __global__ void gla_kernel(const int* __restrict__ seq_off, const int* __restric
                 const int64_t t = tb + j;
                 rq[u] = ld_dt(q, dt, t * ldq + (int64_t)h * dk + i);
                 rk[u] = ld_dt(k, dt, t * ldk + (int64_t)h * dk + i);
-                rz[u] = ld_dt(z, z_dt, t * ldz + (int64_t)h * dk + i) + zbias[h * dk + i];
+                if (!head_decay) rz[u] = ld_dt(z, z_dt, t * ldz + (int64_t)h * dk + i) + zbias[h * dk + i];
             }
         }
 #pragma unroll
@@ -408,8 +412,8 @@ __global__ void gla_kernel(const int* __restrict__ seq_off, const int* __restric
             const int e = threadIdx.x + u * blockDim.x;
             if (e < nt * dk) {
                 sq[e] = rq[u] * qscale;
-                sk[e] = rk[u];
-                sa[e] = expf(inv_tau * log_sigmoid(rz[u]));
+                sk[e] = rk[u] * kscale;
+                sa[e] = head_decay ? head_decay[h] : expf(inv_tau * log_sigmoid(rz[u]));
             }
         }
 #pragma unroll
@@ -465,16 +469,17 @@ __global__ void gla_kernel(const int* __restrict__ seq_off, const int* __restric
 }
 
 extern "C" int mi355_gla_fwd(int n_seq, const int* seq_off, const int* slot, int H, int dk, int dv, const void* q, const void* k, const void* v, const void* z, int dt,
-                             int z_dt, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldz, const float* zbias, float inv_tau, float qscale, float* state, float* o,
-                             void* stream) {
-    MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && seq_off && slot && H > 0 && H <= 65535 && dk > 0 && dk <= 16 * GLA_R && dv > 0 && q && k && v && z && zbias && state && o && dt_ok(dt) && dt_ok(z_dt),
+                             int z_dt, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldz, const float* zbias, float inv_tau, float qscale, const float* head_decay, float kscale,
+                             float* state, float* o, void* stream) {
+    MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && seq_off && slot && H > 0 && H <= 65535 && dk > 0 && dk <= 16 * GLA_R && dv > 0 && q && k && v && state && o && dt_ok(dt),
                   "gla_fwd: bad arguments (key channels per head <= 256)");
-    MI355_REQUIRE(ldq >= (int64_t)H * dk && ldk >= (int64_t)H * dk && ldz >= (int64_t)H * dk && ldv >= (int64_t)H * dv, "gla_fwd: rows too short");
+    MI355_REQUIRE(head_decay || (z && zbias && dt_ok(z_dt) && ldz >= (int64_t)H * dk), "gla_fwd: the decay needs its rows and bias, or a constant per head");
+    MI355_REQUIRE(ldq >= (int64_t)H * dk && ldk >= (int64_t)H * dk && ldv >= (int64_t)H * dv, "gla_fwd: rows too short");
     const int RC = (dk + GLA_R - 1) / GLA_R;
     const size_t lds_bytes = sizeof(float) * ((size_t)3 * GLA_TB * dk + (size_t)GLA_TB * 64 + (size_t)GLA_TB * RC * 64);
     MI355_REQUIRE(lds_bytes <= 64 * 1024, "gla_fwd: LDS budget exceeded");
     gla_kernel<<<dim3(n_seq, H, (dv + 63) / 64), 64 * RC, lds_bytes, ST(stream)>>>(seq_off, slot, H, dk, dv, q, k, v, z, dt, z_dt, ldq, ldk, ldv, ldz, zbias, inv_tau, qscale,
-                                                                                   state, o);
+                                                                                   head_decay, kscale, state, o);
     MI355_LAUNCH_CHECK("gla_fwd");
     return 0;
 }
@@ -528,26 +533,50 @@ extern "C" int mi355_router_logits(int64_t tokens, int E, int K, const float* x,
 // s = sigmoid(logits); choice = s + correction.  Experts form `groups` equal runs of neighbours; a group's score is the sum of its two largest
 // choice scores; only experts of the `keep` best groups may be chosen; the `top` largest allowed choice scores win (ties: lowest index).
 // weights = s of the winners / (their sum + 1e-20) * scale.  One wave per token, expert e on lane e % 64, register e / 64.
+// mode 1 (softmax router): s = softmax(logits) over ALL experts, choice = s (no correction, no groups), weights = s of the winners * scale, not renormalised.
 template <int EPL>
 __global__ __launch_bounds__(256) void moe_route_kernel(int64_t T, int E, int top, int groups, int keep, const float* __restrict__ logits, const float* __restrict__ corr,
-                                                        float scale, int* __restrict__ ids, float* __restrict__ wts) {
+                                                        float scale, int mode, int* __restrict__ ids, float* __restrict__ wts) {
     const int lane = threadIdx.x & 63;
     const float NEG = -__builtin_huge_valf();
     for (int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); t < T; t += (int64_t)gridDim.x * 4) {
         float s[EPL], c[EPL];
+        if (mode == 1) {
+            float mx = NEG;
 #pragma unroll
-        for (int j = 0; j < EPL; ++j) {
-            const int e = lane + 64 * j;
-            if (e < E) {
-                const float zz = logits[t * E + e];
-                s[j] = 1.0f / (1.0f + expf(-zz));
-                c[j] = s[j] + (corr ? corr[e] : 0.f);
-            } else {
-                s[j] = 0.f;
-                c[j] = NEG;
+            for (int j = 0; j < EPL; ++j) {
+                const int e = lane + 64 * j;
+                s[j] = e < E ? logits[t * E + e] : NEG;
+                mx = fmaxf(mx, s[j]);
+            }
+            mx = wave_max(mx);
+            float den = 0.f;
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) {
+                s[j] = lane + 64 * j < E ? expf(s[j] - mx) : 0.f;
+                den += s[j];
+            }
+            den = wave_sum(den);
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) {
+                s[j] = s[j] / den;
+                c[j] = lane + 64 * j < E ? s[j] : NEG;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < EPL; ++j) {
+                const int e = lane + 64 * j;
+                if (e < E) {
+                    const float zz = logits[t * E + e];
+                    s[j] = 1.0f / (1.0f + expf(-zz));
+                    c[j] = s[j] + (corr ? corr[e] : 0.f);
+                } else {
+                    s[j] = 0.f;
+                    c[j] = NEG;
+                }
             }
         }
-        if (groups > 1) {
+        if (mode != 1 && groups > 1) {
             const int per = E / groups;
             // group scores: lane g keeps the score of group g (+ 64 * register)
             float gs[EPL];
@@ -633,7 +662,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int64_t T, int E, int to
                 wts[t * top + n] = sv;
             }
         }
-        const float inv = scale / (wsum + 1e-20f);
+        const float inv = mode == 1 ? scale : scale / (wsum + 1e-20f);
         if (lane < top && lane < 64) {
             ids[t * top + lane] = my_id;
             wts[t * top + lane] = mine * inv;
@@ -643,15 +672,15 @@ __global__ __launch_bounds__(256) void moe_route_kernel(int64_t T, int E, int to
     }
 }
 
-extern "C" int mi355_moe_route(int64_t tokens, int E, int top, int groups, int keep, const float* logits, const float* correction, float scale, int* ids, float* wts,
-                               void* stream) {
-    MI355_REQUIRE(tokens > 0 && E > 0 && E <= 512 && top > 0 && top <= E && logits && ids && wts, "moe_route: bad arguments (experts <= 512)");
+extern "C" int mi355_moe_route(int64_t tokens, int E, int top, int groups, int keep, const float* logits, const float* correction, float scale, int mode, int* ids,
+                               float* wts, void* stream) {
+    MI355_REQUIRE(tokens > 0 && E > 0 && E <= 512 && top > 0 && top <= E && logits && ids && wts && (mode == 0 || mode == 1), "moe_route: bad arguments (experts <= 512)");
     MI355_REQUIRE(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && (int64_t)keep * (E / groups) >= top, "moe_route: the kept groups must hold the experts to choose");
     const int grid = rows_grid(tokens, 4);
-    if (E <= 64) moe_route_kernel<1><<<grid, 256, 0, ST(stream)>>>(tokens, E, top, groups, keep, logits, correction, scale, ids, wts);
-    else if (E <= 128) moe_route_kernel<2><<<grid, 256, 0, ST(stream)>>>(tokens, E, top, groups, keep, logits, correction, scale, ids, wts);
-    else if (E <= 256) moe_route_kernel<4><<<grid, 256, 0, ST(stream)>>>(tokens, E, top, groups, keep, logits, correction, scale, ids, wts);
-    else moe_route_kernel<8><<<grid, 256, 0, ST(stream)>>>(tokens, E, top, groups, keep, logits, correction, scale, ids, wts);
+    if (E <= 64) moe_route_kernel<1><<<grid, 256, 0, ST(stream)>>>(tokens, E, top, groups, keep, logits, correction, scale, mode, ids, wts);
+    else if (E <= 128) moe_route_kernel<2><<<grid, 256, 0, ST(stream)>>>(tokens, E, top, groups, keep, logits, correction, scale, mode, ids, wts);
+    else if (E <= 256) moe_route_kernel<4><<<grid, 256, 0, ST(stream)>>>(tokens, E, top, groups, keep, logits, correction, scale, mode, ids, wts);
+    else moe_route_kernel<8><<<grid, 256, 0, ST(stream)>>>(tokens, E, top, groups, keep, logits, correction, scale, mode, ids, wts);
     MI355_LAUNCH_CHECK("moe_route");
     return 0;
 }

@@ -94,8 +94,9 @@ def latent_kv_append(src, rank, rot, w, eps, pos, dst_row, freq, dims, cache2d):
            L.ptr(cache2d), _dt(cache2d), cache2d.stride(0))
 
 
-def rope_heads(src, H, n, src_hs, src_off, dst, dst_hs, dst_off, rot_start, dims, freq, pos):
-    """dst (fp32) <- n entries per head of src, the pairs of [rot_start, rot_start + dims) rotated by the token's position."""
+def rope_heads(src, H, n, src_hs, src_off, dst, dst_hs, dst_off, rot_start, dims, freq, pos, layout=0):
+    """dst (fp32) <- n entries per head of src, the pairs of [rot_start, rot_start + dims) rotated by the token's position.  ``layout`` 0: neighbouring
+    entries form a pair; 1: entry i pairs with entry i + dims / 2."""
     L.require_gpu(src, dst, freq, pos)
     _rows(src, "rope_heads(src)")
     _rows(dst, "rope_heads(dst)")
@@ -105,7 +106,7 @@ def rope_heads(src, H, n, src_hs, src_off, dst, dst_hs, dst_off, rot_start, dims
     if src.shape[1] < (H - 1) * src_hs + src_off + n or dst.shape[1] < (H - 1) * dst_hs + dst_off + n:
         raise ValueError("rope_heads: rows too short for the head layout")
     L.call("mi355_rope_heads", src.shape[0], H, n, L.ptr(src), _dt(src), src.stride(0), src_hs, src_off, L.ptr(dst), dst.stride(0), dst_hs, dst_off, rot_start, dims,
-           L.ptr(freq), L.ptr(pos))
+           int(layout), L.ptr(freq), L.ptr(pos))
     return dst
 
 
@@ -119,9 +120,15 @@ def gated_headnorm(o, w, gate, H, D, eps, out_dtype):
     return out
 
 
-def gla(q, k, v, z, zbias, inv_tau, qscale, seq_off, slot, state, H, dk, dv):
-    """Gated linear attention over a ragged batch; ``state`` fp32 [slots, H, dk, dv] is read and written at ``slot``.  Returns fp32 [tokens, H * dv]."""
-    L.require_gpu(q, k, v, z, zbias, seq_off, slot, state)
+def gla(q, k, v, z, zbias, inv_tau, qscale, seq_off, slot, state, H, dk, dv, head_decay=None, kscale=1.0):
+    """Gated linear attention over a ragged batch; ``state`` fp32 [slots, H, dk, dv] is read and written at ``slot``.  Returns fp32 [tokens, H * dv].
+    ``head_decay`` (fp32 [H]): a fixed decay per head instead of the per-channel one from ``z`` (``z`` / ``zbias`` may then be None); keys are multiplied
+    by ``kscale``."""
+    L.require_gpu(q, k, v, z, zbias, seq_off, slot, state, head_decay)
+    if head_decay is not None:
+        if head_decay.dtype != F32 or not head_decay.is_contiguous() or head_decay.numel() != H:
+            raise ValueError("gla: head_decay fp32 [H]")
+        return _gla_fixed(q, k, v, head_decay, qscale, kscale, seq_off, slot, state, H, dk, dv)
     for t, n, w in ((q, "q", H * dk), (k, "k", H * dk), (z, "z", H * dk), (v, "v", H * dv)):
         _rows(t, f"gla({n})")
         if t.shape[1] != w or (n != "z" and t.dtype != q.dtype) or t.shape[0] != q.shape[0]:
@@ -133,7 +140,23 @@ def gla(q, k, v, z, zbias, inv_tau, qscale, seq_off, slot, state, H, dk, dv):
         raise ValueError("gla: state fp32 [slots, H, dk, dv], bias fp32 [H * dk]")
     o = torch.empty((q.shape[0], H * dv), dtype=F32, device=q.device)
     L.call("mi355_gla_fwd", n_seq, L.ptr(seq_off), L.ptr(slot), H, dk, dv, L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(z), _dt(q), _dt(z), q.stride(0), k.stride(0), v.stride(0),
-           z.stride(0), L.ptr(zbias), float(inv_tau), float(qscale), L.ptr(state), L.ptr(o))
+           z.stride(0), L.ptr(zbias), float(inv_tau), float(qscale), None, float(kscale), L.ptr(state), L.ptr(o))
+    return o
+
+
+def _gla_fixed(q, k, v, head_decay, qscale, kscale, seq_off, slot, state, H, dk, dv):
+    for t, n, w in ((q, "q", H * dk), (k, "k", H * dk), (v, "v", H * dv)):
+        _rows(t, f"gla({n})")
+        if t.shape[1] != w or t.dtype != q.dtype or t.shape[0] != q.shape[0]:
+            raise ValueError(f"gla({n}): [tokens, {w}] of q's dtype required")
+    n_seq = slot.numel()
+    _i32(seq_off, "gla(seq_off)", n_seq + 1)
+    _i32(slot, "gla(slot)")
+    if state.dtype != F32 or not state.is_contiguous() or tuple(state.shape[1:]) != (H, dk, dv):
+        raise ValueError("gla: state fp32 [slots, H, dk, dv]")
+    o = torch.empty((q.shape[0], H * dv), dtype=F32, device=q.device)
+    L.call("mi355_gla_fwd", n_seq, L.ptr(seq_off), L.ptr(slot), H, dk, dv, L.ptr(q), L.ptr(k), L.ptr(v), None, _dt(q), 0, q.stride(0), k.stride(0), v.stride(0),
+           0, None, 1.0, float(qscale), L.ptr(head_decay), float(kscale), L.ptr(state), L.ptr(o))
     return o
 
 
@@ -148,14 +171,16 @@ def router_logits(x32, w):
     return out
 
 
-def moe_route(logits, correction, top, groups, keep, scale):
+def moe_route(logits, correction, top, groups, keep, scale, softmax=False):
+    """(ids int32 [tokens, top], weights fp32 [tokens, top]).  ``softmax``: scores are the softmax over all experts, the winners' scores times ``scale`` are
+    the weights (not renormalised); otherwise the grouped sigmoid router."""
     L.require_gpu(logits, correction)
     if logits.dtype != F32 or not logits.is_contiguous() or (correction is not None and (correction.dtype != F32 or correction.numel() != logits.shape[1])):
         raise ValueError("moe_route: logits contiguous fp32 [tokens, experts], correction fp32 [experts]")
     T, E = logits.shape
     ids = torch.empty((T, top), dtype=I32, device=logits.device)
     wts = torch.empty((T, top), dtype=F32, device=logits.device)
-    L.call("mi355_moe_route", T, E, top, groups, keep, L.ptr(logits), L.ptr(correction), float(scale), L.ptr(ids), L.ptr(wts))
+    L.call("mi355_moe_route", T, E, top, groups, keep, L.ptr(logits), L.ptr(correction), float(scale), 1 if softmax else 0, L.ptr(ids), L.ptr(wts))
     return ids, wts
 
 
@@ -169,19 +194,22 @@ def moe_dispatch(ids, E):
 
 
 def bgemm(a, b, c, M, N, Kd, batch=1, lda=None, a_bs=0, sbn=None, sbk=1, b_bs=0, ldc=None, c_bs=0, grp_offs=None, a_rows=None, a_div=1, c_rows=None,
-          row_scale=None, epi=0, mfma=None):
+          row_scale=None, epi=0, mfma=None, bias=None):
     """The general strided product (see include/mi355_vlm.h).  Strides default to a's / c's row pitch and b stored [N, K]; the caller vouches that the
     strides stay inside the tensors.  ``mfma`` defaults to bf16 a and b."""
-    L.require_gpu(a, b, c, grp_offs, a_rows, c_rows, row_scale)
+    L.require_gpu(a, b, c, grp_offs, a_rows, c_rows, row_scale, bias)
+    if bias is not None and (bias.dtype != F32 or not bias.is_contiguous() or bias.numel() != N):
+        raise ValueError("bgemm: bias contiguous fp32 [N]")
     if mfma is None:
         mfma = a.dtype == BF16 and b.dtype == BF16
     L.call("mi355_bgemm", batch, M, N, Kd, L.ptr(a), _dt(a), a.stride(0) if lda is None else lda, a_bs, L.ptr(b), _dt(b), b.stride(0) if sbn is None else sbn, sbk, b_bs,
-           L.ptr(c), _dt(c), c.stride(0) if ldc is None else ldc, c_bs, L.ptr(grp_offs), L.ptr(a_rows), a_div, L.ptr(c_rows), L.ptr(row_scale), epi, 1 if mfma else 0)
+           L.ptr(c), _dt(c), c.stride(0) if ldc is None else ldc, c_bs, L.ptr(grp_offs), L.ptr(a_rows), a_div, L.ptr(c_rows), L.ptr(row_scale), epi, 1 if mfma else 0, L.ptr(bias))
     return c
 
 
-def linear(x, w, out_dtype=None):
-    """x [M, K] (bf16 or fp32) times w[N, K]^T (bf16).  bf16 rows go through the MFMA GEMMs (weight stream for <= 8 rows), fp32 rows through the fp32 FMA product."""
+def linear(x, w, out_dtype=None, bias=None):
+    """x [M, K] (bf16 or fp32) times w[N, K]^T (bf16) (+ bias fp32 [N]).  bf16 rows go through the MFMA GEMMs (weight stream for <= 8 rows), fp32 rows through
+    the fp32 FMA product."""
     _rows(x, "linear(x)")
     M, Kd = x.shape
     N = w.shape[0]
@@ -190,14 +218,14 @@ def linear(x, w, out_dtype=None):
     out_dtype = out_dtype or x.dtype
     if x.dtype == BF16:
         aligned = Kd % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
-        if aligned and M <= 8 and out_dtype == BF16:
+        if aligned and M <= 8 and out_dtype == BF16 and bias is None:
             from . import ops_decode
 
             return ops_decode.gemv(x, w)
         if aligned and M > 8:
-            return K.gemm(L.GEMM_NT, x, w, out_dtype=out_dtype)
+            return K.gemm(L.GEMM_NT, x, w, out_dtype=out_dtype, bias=bias)
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
-    return bgemm(x, w, out, M, N, Kd)
+    return bgemm(x, w, out, M, N, Kd, bias=bias)
 
 
 def attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys):
@@ -209,9 +237,11 @@ def attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys):
     return max(1, min(-(-max_keys // 256), 32, 256 // tiles))
 
 
-def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, desc, max_new, scale, max_keys=0):
+def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, desc, max_new, scale, max_keys=0, kv_rep=1, window=0, keep_first=0):
     """Two-part-key causal attention over a ragged batch.  ``desc`` = (q_row0, n_new, past, k1_row0, k2_row0, v_row0) int32 [n_seq] each.  ``max_keys``
-    (the longest sequence's keys, if the caller knows it) lets one-token steps over long caches spread a tile's keys over several workgroups."""
+    (the longest sequence's keys, if the caller knows it) lets one-token steps over long caches spread a tile's keys over several workgroups.
+    ``kv_rep``: query heads per key / value head (strides per key / value head).  ``window`` > 0: a query sees a key only ``window`` positions back, or
+    among the first ``keep_first`` of the sequence."""
     L.require_gpu(q, k1, k2, v, out, *desc)
     for t, n in ((q, "q"), (k1, "k1"), (v, "v"), (out, "out")):
         _rows(t, f"latent_attn({n})")
@@ -222,7 +252,7 @@ def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, d
         _i32(t, "latent_attn(desc)", n_seq)
     mfma = v.dtype == BF16
     splits, ws = 1, None
-    if mfma and D1 + D2 <= 320 and DV <= 256 and max_keys:
+    if mfma and D1 + D2 <= 320 and DV <= 256 and max_keys and not window:
         head_tiles = -(-H // hm)
         splits = attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys)
         if splits > 1:
@@ -230,5 +260,116 @@ def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, d
             ws = torch.empty(n_seq * head_tiles * -(-max_new * hm // 128) * splits * 128 * (2 + dvp), dtype=F32, device=v.device)
     L.call("mi355_latent_attn", n_seq, max_new, H, hm, D1, D2, DV, L.ptr(q), q.stride(0), q_hs, L.ptr(k1), k1.stride(0), k1_hs, L.ptr(k2), 0 if k2 is None else k2.stride(0),
            L.ptr(v), v.stride(0), v_hs, L.ptr(out), out.stride(0), o_hs, _dt(v), *[L.ptr(t) for t in desc], float(scale), 1 if mfma else 0, splits, L.ptr(ws),
-           0 if ws is None else ws.numel())
+           0 if ws is None else ws.numel(), int(kv_rep), int(window), int(keep_first))
+    return out
+
+
+def group_rmsnorm_sum(x, groups, eps, y1=None, y2=None, parts=1, x_out=None, norm_a=None, norm_b=None):
+    """v = x + y1 + (sum of y2's ``parts`` rows per token) on fp32 rows; ``x_out`` (True: a new tensor, or a tensor, or None) receives v.  ``norm_a`` /
+    ``norm_b`` = (weight fp32 [width], dtype or None, want_fp32_copy): RMS norm of v in ``groups`` equal consecutive groups times the weight.
+    Returns (x_out or None, (a, a32), (b, b32))."""
+    L.require_gpu(x, y1, y2)
+    _rows(x, "group_rmsnorm_sum(x)")
+    T, width = x.shape
+    if x.dtype != F32 or not x.is_contiguous():
+        raise ValueError("group_rmsnorm_sum: x contiguous fp32 [tokens, width]")
+    for y, n, rows in ((y1, "y1", T), (y2, "y2", T * parts)):
+        if y is not None:
+            _rows(y, f"group_rmsnorm_sum({n})")
+            if tuple(y.shape) != (rows, width):
+                raise ValueError(f"group_rmsnorm_sum({n}): [{rows}, {width}] required, got {tuple(y.shape)}")
+    if x_out is True:
+        x_out = torch.empty_like(x)
+    outs, args = [], []
+    for nm in (norm_a, norm_b):
+        if nm is None:
+            outs.append((None, None))
+            args += [None, None, 0, None]
+            continue
+        w, dtype, want32 = nm
+        if w.dtype != F32 or w.numel() != width or not w.is_contiguous():
+            raise ValueError("group_rmsnorm_sum: weight fp32 [width]")
+        o = torch.empty((T, width), dtype=dtype, device=x.device) if dtype is not None else None
+        o32 = o if dtype == F32 and want32 else (torch.empty((T, width), dtype=F32, device=x.device) if want32 else None)
+        outs.append((o, o32))
+        args += [L.ptr(w), L.ptr(o), 0 if o is None else _dt(o), None if o32 is o else L.ptr(o32)]
+    L.call("mi355_group_rmsnorm_sum", T, width, L.ptr(x), L.ptr(y1), 0 if y1 is None else _dt(y1), 0 if y1 is None else y1.stride(0), L.ptr(y2),
+           0 if y2 is None else _dt(y2), 0 if y2 is None else y2.stride(0), int(parts), L.ptr(x_out), int(groups), float(eps), *args)
+    return x_out, outs[0], outs[1]
+
+
+def ragged_conv(x, w, state, row_seq, seq_off, slot, act=False, residual=False, out_dtype=None):
+    """Causal convolution over time on every channel of the packed rows ``x`` [tokens, C], w fp32 [C, taps]; ``state`` fp32 [slots, taps - 1, C] carries a
+    sequence's last inputs from step to step (read, then updated).  y = (x if residual) + (silu if act)(conv)."""
+    L.require_gpu(x, w, state, row_seq, seq_off, slot)
+    _rows(x, "ragged_conv(x)")
+    T, C = x.shape
+    taps = w.shape[1]
+    n_seq = slot.numel()
+    if w.dtype != F32 or not w.is_contiguous() or w.shape[0] != C:
+        raise ValueError("ragged_conv: weight contiguous fp32 [C, taps]")
+    if taps > 1 and (state is None or state.dtype != F32 or not state.is_contiguous() or tuple(state.shape[1:]) != (taps - 1, C)):
+        raise ValueError("ragged_conv: state contiguous fp32 [slots, taps - 1, C]")
+    _i32(row_seq, "ragged_conv(row_seq)", T)
+    _i32(seq_off, "ragged_conv(seq_off)", n_seq + 1)
+    _i32(slot, "ragged_conv(slot)")
+    y = torch.empty((T, C), dtype=out_dtype or x.dtype, device=x.device)
+    L.call("mi355_ragged_conv", T, n_seq, C, taps, L.ptr(x), _dt(x), x.stride(0), L.ptr(w), L.ptr(row_seq), L.ptr(seq_off), L.ptr(slot), L.ptr(state), 1 if act else 0,
+           1 if residual else 0, L.ptr(y), _dt(y), y.stride(0))
+    return y
+
+
+def qkv_rows_append(src, H, G, d, dv, bias, qw, kw, eps, qscale, dims, layout, freq, pos, dst_row, cache2d):
+    """Rows [H x d | G x d | G x dv] -> fp32 queries [tokens, H * d] (bias, head norm, rotation, per-head scale) and key / value rows of ``cache2d``."""
+    L.require_gpu(src, bias, qw, kw, qscale, freq, pos, dst_row, cache2d)
+    _rows(src, "qkv_rows_append(src)")
+    _rows(cache2d, "qkv_rows_append(cache)")
+    T = src.shape[0]
+    if src.shape[1] != (H + G) * d + G * dv or cache2d.shape[1] != G * (d + dv):
+        raise ValueError("qkv_rows_append: row widths do not match the head layout")
+    for t, n in ((bias, (H + G) * d + G * dv), (qw, d), (kw, d), (qscale, H), (freq, dims // 2)):
+        if t is not None and (t.dtype != F32 or not t.is_contiguous() or t.numel() < n):
+            raise ValueError("qkv_rows_append: vectors are contiguous fp32 of the layout's sizes")
+    _i32(pos, "qkv_rows_append(pos)", T)
+    _i32(dst_row, "qkv_rows_append(dst_row)", T)
+    q = torch.empty((T, H * d), dtype=F32, device=src.device)
+    L.call("mi355_qkv_rows_append", T, H, G, d, dv, L.ptr(src), _dt(src), src.stride(0), L.ptr(bias), L.ptr(qw), L.ptr(kw), float(eps), L.ptr(qscale), int(dims), int(layout),
+           L.ptr(freq), L.ptr(pos), L.ptr(dst_row), L.ptr(q), q.stride(0), L.ptr(cache2d), _dt(cache2d), cache2d.stride(0))
+    return q
+
+
+def delta_rule(q, k, v, b, a, A_log, dt_bias, qscale, seq_off, slot, state, H, G, dk, dv):
+    """Gated delta rule over a ragged batch (raw q / k rows: made unit vectors inside); ``state`` fp32 [slots, H, dk, dv].  Returns fp32 [tokens, H * dv]."""
+    L.require_gpu(q, k, v, b, a, A_log, dt_bias, seq_off, slot, state)
+    T = q.shape[0]
+    for t, n, w in ((q, "q", G * dk), (k, "k", G * dk), (v, "v", H * dv), (b, "b", H), (a, "a", H)):
+        _rows(t, f"delta_rule({n})")
+        if t.shape != (T, w):
+            raise ValueError(f"delta_rule({n}): [tokens, {w}] required")
+    if q.dtype != k.dtype or b.dtype != a.dtype:
+        raise ValueError("delta_rule: q / k share a dtype, so do b / a")
+    n_seq = slot.numel()
+    _i32(seq_off, "delta_rule(seq_off)", n_seq + 1)
+    _i32(slot, "delta_rule(slot)")
+    if state.dtype != F32 or not state.is_contiguous() or tuple(state.shape[1:]) != (H, dk, dv):
+        raise ValueError("delta_rule: state fp32 [slots, H, dk, dv]")
+    for t in (A_log, dt_bias):
+        if t.dtype != F32 or t.numel() != H or not t.is_contiguous():
+            raise ValueError("delta_rule: A_log and dt_bias fp32 [H]")
+    o = torch.empty((T, H * dv), dtype=F32, device=q.device)
+    L.call("mi355_delta_rule_ragged", n_seq, L.ptr(seq_off), L.ptr(slot), H, G, dk, dv, L.ptr(q), L.ptr(k), _dt(q), q.stride(0), k.stride(0), L.ptr(v), _dt(v), v.stride(0),
+           L.ptr(b), L.ptr(a), _dt(b), b.stride(0), a.stride(0), L.ptr(A_log), L.ptr(dt_bias), float(qscale), L.ptr(state), L.ptr(o))
+    return o
+
+
+GLU_GELU_TANH, GLU_CLAMPED_SWISH = 0, 1
+
+
+def glu_rows(x, kind, limit=0.0, out_dtype=None):
+    """Rows [gate | up] -> act(gate) * up: ``GLU_GELU_TANH``, or ``GLU_CLAMPED_SWISH`` (g = min(gate, limit), u = clamp(up, +-limit), g sigmoid(1.702 g) (u + 1))."""
+    L.require_gpu(x)
+    _rows(x, "glu_rows(x)")
+    F = x.shape[1] // 2
+    out = torch.empty((x.shape[0], F), dtype=out_dtype or x.dtype, device=x.device)
+    L.call("mi355_glu_rows", x.shape[0], F, L.ptr(x), _dt(x), x.stride(0), int(kind), float(limit), L.ptr(out), _dt(out), out.stride(0))
     return out

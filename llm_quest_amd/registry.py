@@ -28,7 +28,14 @@ def _gemepel(model_dir, act_dtype, device):
     return load_gemepel(model_dir, act_dtype, device)
 
 
+def _mepatar(model_dir, act_dtype, device):
+    from llm_quest_amd.mepatar.mepatar_weight_loading import load_mepatar
+
+    return load_mepatar(model_dir, act_dtype, device)
+
+
 register("Gemepel", _gemepel)
+register("Mepatar", _mepatar)
 
 
 def load_model(model_dir, dtype="bfloat16", device="cuda"):

@@ -147,6 +147,8 @@ class SlotStateCache:
         row ``slot * capacity + position`` of the 2-D view ``rows2d(i)`` is what the kernels address;
       * ``("shared", j)``    -- the layer reads layer j's rows and stores nothing;
       * ``("state", shape)`` -- a fixed-size fp32 state ``[slots, *shape]`` (the matrix state of linear attention), zeroed when a slot is opened;
+      * ``{"rows": width or None, "states": {name: shape}}`` -- both at once, with several named fp32 states (``state(i, name)``): a layer that caches
+        key / value rows and carries the last inputs of short convolutions, or a recurrent state next to its convolutions' inputs;
       * ``None``             -- nothing.
     Besides, per slot: the length so far and the last token (the embedding of some designs looks one token back).  Growth follows ``KVCache``: the row
     capacity starts at what the first sequences need plus ``initial_chunk_size`` and grows by whole ``chunk_size`` steps up to ``context_len``; slots double."""
@@ -160,6 +162,7 @@ class SlotStateCache:
         self.capacity = min(self.context_len, int(capacity))
         self.rows = [None] * len(self.layer_specs)
         self.states = [None] * len(self.layer_specs)
+        self.named = [{} for _ in self.layer_specs]  # layer -> name -> fp32 [slots, *shape]
         self.length = [0] * self.slots
         self.last_token = [-1] * self.slots
         self._slot_of = {}
@@ -167,18 +170,28 @@ class SlotStateCache:
         self.reuses = 0  # slots handed out again after a close (bookkeeping for tests / logs)
         self._used_once = set()
         for i, spec in enumerate(self.layer_specs):
-            if spec is not None and spec[0] == "state":
+            if spec is not None and not isinstance(spec, dict) and spec[0] == "state":
                 self.states[i] = torch.zeros((self.slots,) + tuple(spec[1]), dtype=torch.float32, device=device)
+            elif isinstance(spec, dict):
+                for name, shape in (spec.get("states") or {}).items():
+                    self.named[i][name] = torch.zeros((self.slots,) + tuple(shape), dtype=torch.float32, device=device)
         if self.capacity:
             self._allocate_rows(self.capacity)
 
     # ------------------------------------------------------------------ storage
+    @staticmethod
+    def _row_width(spec):
+        if isinstance(spec, dict):
+            return spec.get("rows") or 0
+        return spec[1] if spec is not None and spec[0] == "rows" else 0
+
     def _allocate_rows(self, capacity):
         for i, spec in enumerate(self.layer_specs):
-            if spec is None or spec[0] != "rows":
+            width = self._row_width(spec)
+            if not width:
                 continue
             old = self.rows[i]
-            new = torch.zeros((self.slots, capacity, spec[1]), dtype=self.dtype, device=self.device)
+            new = torch.zeros((self.slots, capacity, width), dtype=self.dtype, device=self.device)
             if old is not None:
                 n = min(old.shape[0], self.slots)
                 new[:n, : old.shape[1]].copy_(old[:n])
@@ -194,6 +207,9 @@ class SlotStateCache:
         for i, st in enumerate(self.states):
             if st is not None:
                 self.states[i] = torch.cat([st, torch.zeros_like(st)], dim=0)
+        for d in self.named:
+            for name, st in d.items():
+                d[name] = torch.cat([st, torch.zeros_like(st)], dim=0)
         if self.capacity:
             self._allocate_rows(self.capacity)
 
@@ -227,6 +243,9 @@ class SlotStateCache:
         for st in self.states:
             if st is not None:
                 st[slot].zero_()
+        for d in self.named:
+            for st in d.values():
+                st[slot].zero_()
         return slot
 
     def slot(self, seq_id):
@@ -250,14 +269,14 @@ class SlotStateCache:
     # ------------------------------------------------------------------ views for the kernels
     def source(self, layer_idx):
         spec = self.layer_specs[layer_idx]
-        return spec[1] if spec is not None and spec[0] == "shared" else layer_idx
+        return spec[1] if spec is not None and not isinstance(spec, dict) and spec[0] == "shared" else layer_idx
 
     def rows2d(self, layer_idx):
         r = self.rows[self.source(layer_idx)]
         return r.view(r.shape[0] * r.shape[1], r.shape[2])
 
-    def state(self, layer_idx):
-        return self.states[layer_idx]
+    def state(self, layer_idx, name=None):
+        return self.states[layer_idx] if name is None else self.named[layer_idx][name]
 
 
 # ----------------------------------------------------------------------------------------------- checkpoint import (row f2)
