@@ -95,14 +95,15 @@ def visible(i, j, size, keep_first):
     return j <= i and (i - j < size or j < keep_first)
 
 
-def window_attention(q, k, v, scale, temp, size, keep_first):
-    """q [T, H, d], k [T, G, d], v [T, G, dv]; query head h reads key/value head h // (H/G); softmax over the visible keys."""
+def window_attention(q, k, v, scale, temp, size, keep_first, first_query=0):
+    """q [T, H, d], k [T, G, d], v [T, G, dv]; query head h reads key/value head h // (H/G); softmax over the visible keys.  Rows before
+    ``first_query`` are left zero (a caller that only needs the last queries)."""
     T, H, d = q.shape
     G, dv = k.shape[1], v.shape[-1]
     out = torch.zeros(T, H, dv, dtype=q.dtype)
     for h in range(H):
         g = h // (H // G)
-        for i in range(T):
+        for i in range(first_query, T):
             js = [j for j in range(i + 1) if visible(i, j, size, keep_first)]
             s = torch.stack([(q[i, h] * k[j, g]).sum() for j in js]) * scale * temp[h]
             p = torch.softmax(s, dim=0)

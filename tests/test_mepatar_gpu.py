@@ -1,0 +1,493 @@
+"""GPU tests of the Mepatar serving path against the plain oracle (oracle/mepatar.py): each mechanism's kernel alone, then the model through the
+registry, the slot cache and the ragged-batch scheduler -- whole prompts, token-by-token decoding, portions, unequal batches, reused slots, keys at the
+window's and the kept tokens' edges, odd sizes, greedy generation.  fp32 mode is held to fp32 rounding; bf16 mode to a few bf16 roundings of the
+logits' scale."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import mepatar as O
+from tests import mepatar_util as U
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+F32, F64, BF16, I32 = torch.float32, torch.float64, torch.bfloat16, torch.int32
+
+
+def dev_i32(x):
+    return torch.tensor(x, dtype=I32).to(DEV)
+
+
+def row_err(got, want, quantile=None):
+    """Per row: rms of the difference (mean removed) over the rms of the wanted rows; the worst row, or a quantile of the rows (bf16 model runs are
+    judged on the median row: a token whose two best experts lie within a bf16 rounding may legitimately take the other one)."""
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    e = d.pow(2).mean(-1).sqrt() / want.pow(2).mean().sqrt()
+    return e.max().item() if quantile is None else torch.quantile(e, quantile).item()
+
+
+def model_err(got, want, dt):
+    return row_err(got, want, None if dt == "float32" else 0.5)
+
+
+TOL = {"float32": 3e-5, "bfloat16": 6e-2}
+
+
+@pytest.fixture(scope="module")
+def checkpoint(tmp_path_factory):
+    cfg = U.make_config(U.default_layers())
+    w = U.make_weights(cfg, 11)
+    return U.save(str(tmp_path_factory.mktemp("mepatar")), cfg, w), cfg, w
+
+
+@pytest.fixture(scope="module")
+def models(checkpoint):
+    from llm_quest_amd import registry
+
+    folder, cfg, w = checkpoint
+    return {dt: registry.load_model(folder, dt, DEV) for dt in ("float32", "bfloat16")}, cfg, w
+
+
+def tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+_oracle_cache = {}
+
+
+def oracle(cfg, w, toks, layers=False):
+    key = (id(w), tuple(toks), layers)
+    if key not in _oracle_cache:
+        _oracle_cache[key] = O.forward(toks, w, cfg, F64, return_layers=layers)
+    return _oracle_cache[key]
+
+
+def batch_of(model, **kw):
+    from llm_quest_amd.generate import RaggedBatch
+
+    return RaggedBatch(model, **kw)
+
+
+# ------------------------------------------------------------------------------------------------------------------- the model through the scheduler
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_whole_prompt_every_layer(models, dt):
+    ms, cfg, w = models
+    toks = tokens(70, cfg["vocab"], 1)
+    want, layers = oracle(cfg, w, toks, layers=True)
+    b = batch_of(ms[dt])
+    got, got_layers = b.step([("a", toks)], [list(range(len(toks)))], return_layers=True)
+    assert len(got_layers) == len(layers)
+    for i, l in enumerate(got_layers):
+        assert model_err(l, layers[i], dt) < (3e-5 if dt == "float32" else 8e-2), f"residual stream after layer {i}"
+    assert model_err(got, want, dt) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_token_by_token_from_the_first_token(models, dt):
+    """Every token alone: the first one meets empty states and zeros before the sequence's start in every convolution."""
+    ms, cfg, w = models
+    toks = tokens(45, cfg["vocab"], 2)
+    want = oracle(cfg, w, toks)
+    b = batch_of(ms[dt])
+    got = torch.cat([b.step([("a", [t])]) for t in toks])
+    assert model_err(got, want, dt) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_portions_of_several_sizes(models, dt):
+    """Portions shorter than the convolutions' reach (1 and 2 tokens) keep older inputs in the carried state."""
+    ms, cfg, w = models
+    toks = tokens(90, cfg["vocab"], 3)
+    want = oracle(cfg, w, toks)
+    b = batch_of(ms[dt])
+    got, at = [], 0
+    for n in [7, 2, 2, 1, 33, 1, 9, 2, 33]:
+        got.append(b.step([("a", toks[at : at + n])], [list(range(n))]))
+        at += n
+    assert at == len(toks)
+    assert model_err(torch.cat(got), want, dt) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_unequal_batch_equals_each_request_alone(models, dt):
+    ms, cfg, w = models
+    lens, tail = [1, 41, 17, 66], 9
+    seqs = [tokens(n + tail, cfg["vocab"], 10 + i) for i, n in enumerate(lens)]
+    alone = []
+    for s in seqs:
+        b = batch_of(ms[dt])
+        alone.append(b.step([("x", s)], [list(range(len(s)))]))
+    b = batch_of(ms[dt], slots=2)  # fewer slots than sequences: the cache grows
+    got = [[] for _ in seqs]
+    out = b.step([(i, s[: lens[i]]) for i, s in enumerate(seqs)], [list(range(n)) for n in lens])
+    at = 0
+    for i, n in enumerate(lens):
+        got[i].append(out[at : at + n])
+        at += n
+    live = list(range(len(seqs)))
+    for k in range(tail):
+        if k == 4:  # two requests leave early; the others go on
+            for i in (0, 2):
+                b.finish(i)
+                live.remove(i)
+        out = b.step([(i, [seqs[i][lens[i] + k]]) for i in live])
+        for j, i in enumerate(live):
+            got[i].append(out[j : j + 1])
+    for i, s in enumerate(seqs):
+        g = torch.cat(got[i])
+        ref = alone[i][: g.shape[0]]
+        assert model_err(g, ref, dt) < (1e-5 if dt == "float32" else 3e-2), f"request {i} in the batch differs from the request alone"
+        assert model_err(g, oracle(cfg, w, s)[: g.shape[0]], dt) < TOL[dt]
+
+
+def test_freed_slots_are_reused_without_leftovers(models):
+    """A long sequence leaves rows, recurrent state and convolution inputs behind; the next, shorter one takes its slot and must see none of it.  The
+    cache starts small, so the rows also grow while a sequence is alive."""
+    ms, cfg, w = models
+    b = batch_of(ms["float32"], slots=1)
+    b.cache.initial_chunk_size, b.cache.chunk_size = 4, 8
+    long_, short = tokens(60, cfg["vocab"], 20), tokens(21, cfg["vocab"], 21)
+    b.step([("long", long_[:50])])
+    for t in long_[50:]:
+        b.step([("long", [t])])
+    b.finish("long")
+    got = [b.step([("short", short[:12])], [list(range(12))])] + [b.step([("short", [t])]) for t in short[12:]]
+    assert b.cache.reuses >= 1 and b.cache.slots == 1
+    assert row_err(torch.cat(got), oracle(cfg, w, short)) < TOL["float32"]
+
+
+def test_long_decoding_passes_the_windows(models):
+    """Decoded tokens walk past both windows (20 and 7 keys) and far past the kept first tokens."""
+    ms, cfg, w = models
+    toks = tokens(200, cfg["vocab"], 30)
+    b = batch_of(ms["float32"])
+    b.step([("a", toks[:5])])
+    got = torch.cat([b.step([("a", [t])]) for t in toks[5:]])
+    assert row_err(got, oracle(cfg, w, toks)[5:]) < TOL["float32"]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_other_sizes_odd_and_one(tmp_path, dt):
+    """Sizes that are no multiples of 8 or of each other's, one head, one group, one tap, top 1, more than 64 experts, a window of one key, a window that
+    never closes, three and four query heads per key head, delta heads that share query / key heads, a key width over several register chunks."""
+    from llm_quest_amd import registry
+
+    layers = [(U.retention(heads=1, dim=10, vdim=70, decay=[0.93], rot_dims=0), U.moe(experts=5, top=1, ff=18, limit=0.5)),
+              (U.attention(heads=6, kv_heads=2, dim=12, vdim=20, size=1, keep_first=2, rot_dims=4), U.moe(experts=70, top=6, ff=10, limit=3.0)),
+              (U.delta(heads=6, kv_heads=2, dim=36, vdim=12, conv=1), None),
+              (U.attention(heads=4, kv_heads=1, dim=20, vdim=36, size=1000, keep_first=0, rot_dims=20, scale=0.4), U.dense(ff=30)),
+              (U.delta(heads=1, kv_heads=1, dim=100, vdim=68, conv=5), U.moe(experts=4, top=4, ff=30, limit=1.0)),
+              (U.retention(heads=5, dim=36, vdim=12, rot_dims=36, base=77.0), U.dense(ff=44))]
+    cfg = U.make_config(layers, width=100, vocab=77, eps=1e-6, groups=1, taps=1, embed_scale=1.0)
+    w = U.make_weights(cfg, 5)
+    model = registry.load_model(U.save(str(tmp_path), cfg, w), dt, DEV)
+    toks = tokens(40, cfg["vocab"], 6)
+    want = O.forward(toks, w, cfg, F64)
+    b = batch_of(model)
+    got = [b.step([("a", toks[:29])], [list(range(29))])] + [b.step([("a", [t])]) for t in toks[29:]]
+    assert model_err(torch.cat(got), want, dt) < TOL[dt]
+
+
+def test_wide_rows_many_groups_long_taps(tmp_path):
+    """A row wider than 512 in 5 groups, 6 taps, key widths 128 and 200."""
+    from llm_quest_amd import registry
+
+    layers = [(U.delta(heads=2, kv_heads=1, dim=128, vdim=64, conv=3), U.dense(ff=64)),
+              (U.retention(heads=2, dim=200, vdim=24), None),
+              (U.attention(heads=2, kv_heads=2, dim=136, vdim=72, size=9, keep_first=4, rot_dims=64), U.moe(experts=3, top=2, ff=16, limit=1.0))]
+    cfg = U.make_config(layers, width=520, vocab=50, groups=5, taps=6)
+    w = U.make_weights(cfg, 9)
+    toks = tokens(30, cfg["vocab"], 8)
+    want = O.forward(toks, w, cfg, F64)
+    for dt in ("float32", "bfloat16"):
+        model = registry.load_model(U.save(str(tmp_path / dt), cfg, w), dt, DEV)
+        b = batch_of(model)
+        got = [b.step([("a", toks[:21])], [list(range(21))])] + [b.step([("a", [t])]) for t in toks[21:]]
+        assert model_err(torch.cat(got), want, dt) < TOL[dt]
+
+
+def test_greedy_generation_through_the_entry_point(models):
+    from llm_quest_amd.generate import generate_ragged
+
+    ms, cfg, w = models
+    prompts = [tokens(n, cfg["vocab"], 40 + n) for n in (4, 19, 9)]
+    out = generate_ragged(ms["float32"], prompts, max_gen=10)
+    for p, gen in zip(prompts, out):
+        assert len(gen) == 10
+        seq = list(p)
+        for t in gen:
+            lg = O.forward(seq, w, cfg, F64)[-1]
+            top = torch.topk(lg, 2)
+            if int(top.indices[0]) != t:
+                assert float(top.values[0] - top.values[1]) < 1e-4, "greedy token differs from the oracle's without a near tie"
+                break
+            seq.append(t)
+    first = out[1][2]
+    out2 = generate_ragged(ms["float32"], prompts, max_gen=10, eos_ids=[first])
+    assert out2[1] == out[1][: out[1].index(first)] and out2[0][: len(out2[0])] == out[0][: len(out2[0])]
+
+
+# ------------------------------------------------------------------------------------------------------------------- mechanisms alone
+class _Slots:
+    """The descriptors of a step over sequences that each own one slot."""
+
+    def __init__(self, lens, slots=None):
+        off = [0]
+        for n in lens:
+            off.append(off[-1] + n)
+        self.seq_off = dev_i32(off)
+        self.slots = dev_i32(list(range(len(lens))) if slots is None else slots)
+        self.row_seq = dev_i32([i for i, n in enumerate(lens) for _ in range(n)])
+        self.off = off
+
+
+@pytest.mark.parametrize("width,groups", [(72, 3), (100, 1), (520, 5), (2048, 2), (1000, 8)])
+def test_group_norm_with_the_residual_sum(width, groups):
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(width)
+    T, parts = 9, 3
+    x, y1, y2 = torch.randn(T, width, generator=g) * 3, torch.randn(T, width, generator=g), torch.randn(T * parts, width, generator=g)
+    wa, wb = torch.rand(width, generator=g) + 0.5, torch.rand(width, generator=g) + 0.5
+    x_out, (a, a32), (b, b32) = S.group_rmsnorm_sum(x.to(DEV), groups, 1e-5, y1=y1.to(DEV).to(BF16), y2=y2.to(DEV), parts=parts, x_out=True, norm_a=(wa.to(DEV), None, True),
+                                                    norm_b=(wb.to(DEV), BF16, True))
+    v = x.double() + y1.to(BF16).double() + y2.double().reshape(T, parts, width).sum(1)
+    assert a is None and torch.allclose(x_out.cpu().double(), v, atol=1e-5)
+    assert row_err(a32, O.group_rms_norm(v, wa.double(), groups, 1e-5)) < 2e-6
+    assert row_err(b32, O.group_rms_norm(v, wb.double(), groups, 1e-5)) < 2e-6
+    assert torch.equal(b.cpu(), b32.cpu().to(BF16))
+    # a group that is tiny next to the others must be normed by its own size
+    x2 = torch.randn(T, width, generator=g)
+    x2[:, : width // groups] *= 1e-3
+    _, (n, _), _ = S.group_rmsnorm_sum(x2.to(DEV), groups, 1e-12, norm_a=(wa.to(DEV), F32, False))
+    assert row_err(n, O.group_rms_norm(x2.double(), wa.double(), groups, 1e-12)) < 2e-6
+
+
+@pytest.mark.parametrize("taps", [1, 2, 4, 7])
+def test_short_convolution_carries_its_inputs_over_cuts(taps):
+    """Two sequences of different lengths, cut into portions of 1, 2 and more tokens, against the whole-sequence convolution, with and without the
+    activation and the added input."""
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(taps)
+    C = 70
+    w = torch.randn(C, taps, generator=g)
+    seqs = [torch.randn(23, C, generator=g), torch.randn(11, C, generator=g)]
+    for act, res in ((False, True), (True, False)):
+        state = torch.zeros(2, taps - 1, C, device=DEV) if taps > 1 else None
+        at, got = [0, 0], [[], []]
+        for cut in ([1, 1], [2, 1], [1, 2], [5, 3], [14, 4]):
+            d = _Slots(cut)
+            x = torch.cat([seqs[i][at[i] : at[i] + cut[i]] for i in range(2)]).to(DEV)
+            y = S.ragged_conv(x, w.to(DEV), state, d.row_seq, d.seq_off, d.slots, act=act, residual=res)
+            for i in range(2):
+                got[i].append(y[d.off[i] : d.off[i + 1]])
+                at[i] += cut[i]
+        for i in range(2):
+            c = O.causal_conv(seqs[i].double(), w.double())
+            want = (O.silu(c) if act else c) + (seqs[i].double() if res else 0)
+            assert row_err(torch.cat(got[i]), want) < 2e-6
+
+
+@pytest.mark.parametrize("layout", ["half", "interleaved"])
+def test_rotary_layouts_at_large_positions(layout):
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(3)
+    H, d, dims, base = 3, 20, 12, 1e6
+    pos = [0, 1, 2, 63, 64, 1000, 99999]
+    x = torch.randn(len(pos), H, d, generator=g)
+    full = torch.zeros(pos[-1] + 1, H, d, dtype=F64)
+    full[pos] = x.double()
+    want = O.rotary(full, dims, base, layout)[pos]
+    out = torch.empty(len(pos), H * d, dtype=F32, device=DEV)
+    S.rope_heads(x.reshape(len(pos), H * d).to(DEV), H, d, d, 0, out, d, 0, 0, dims, S.rope_frequencies(dims, base, DEV), dev_i32(pos), layout=1 if layout == "half" else 0)
+    # the angle position x frequency is an fp32 product: at position 1e5 it is good to ~1e-2 / 2^-7 rad, at small positions to rounding
+    assert row_err(out[:5], want.reshape(len(pos), H * d)[:5]) < 1e-5
+    assert row_err(out, want.reshape(len(pos), H * d)) < 3e-4
+
+
+@pytest.mark.parametrize("dk,dv", [(24, 40), (32, 64), (200, 72)])
+def test_retention_carries_state_over_cuts_and_keeps_a_far_token(dk, dv):
+    """A token far back whose key matches the last query and whose value is large must come through with decay^distance."""
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(dk)
+    H, T = 2, 150
+    decay = [0.999, 0.9]
+    q, k, v = torch.randn(T, H, dk, generator=g), torch.randn(T, H, dk, generator=g), torch.randn(T, H, dv, generator=g)
+    k[3], q[T - 1], v[3] = q[T - 1] * 3, q[T - 1], v[3] * 50
+    want = O.retention(q.double(), k.double() * dk ** -0.5, v.double(), decay)
+    state = torch.zeros(1, H, dk, dv, device=DEV)
+    got, at = [], 0
+    for n in [1, 2, 7, 8, 9, 64, 58, 1]:
+        d = _Slots([n])
+        sl = slice(at, at + n)
+        got.append(S.gla(q[sl].reshape(n, -1).to(DEV), k[sl].reshape(n, -1).to(DEV), v[sl].reshape(n, -1).to(DEV), None, None, 1.0, 1.0, d.seq_off, d.slots, state, H, dk, dv,
+                         head_decay=torch.tensor(decay, device=DEV), kscale=dk ** -0.5))
+        at += n
+    assert at == T
+    assert row_err(torch.cat(got), want.reshape(T, -1)) < 3e-5  # fp32 sums over up to 200 key channels next to a value 50 times the others
+
+
+@pytest.mark.parametrize("dk,dv,H,G", [(24, 40, 4, 2), (32, 32, 2, 2), (128, 72, 2, 1), (200, 16, 3, 3)])
+def test_delta_rule_carries_state_over_cuts(dk, dv, H, G):
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(dk + H)
+    lens = [60, 17]
+    A_log, dt_bias = torch.randn(H, generator=g) - 1.0, torch.randn(H, generator=g) * 0.5
+    data = []
+    for T in lens:
+        data.append(dict(q=torch.randn(T, G, dk, generator=g), k=torch.randn(T, G, dk, generator=g), v=torch.randn(T, H, dv, generator=g), b=torch.randn(T, H, generator=g) * 2,
+                         a=torch.randn(T, H, generator=g) * 2))
+    state = torch.zeros(2, H, dk, dv, device=DEV)
+    got, at = [[], []], [0, 0]
+    for cut in ([1, 1], [2, 1], [9, 8], [31, 2], [17, 5]):
+        d = _Slots(cut)
+        cat = {n: torch.cat([data[i][n][at[i] : at[i] + cut[i]].reshape(cut[i], -1) for i in range(2)]).to(DEV) for n in "qkvba"}
+        o = S.delta_rule(cat["q"], cat["k"], cat["v"], cat["b"], cat["a"], A_log.to(DEV), dt_bias.to(DEV), dk ** -0.5, d.seq_off, d.slots, state, H, G, dk, dv)
+        for i in range(2):
+            got[i].append(o[d.off[i] : d.off[i + 1]])
+            at[i] += cut[i]
+    for i, T in enumerate(lens):
+        x = {n: t.double() for n, t in data[i].items()}
+        q = x["q"] / torch.sqrt((x["q"] ** 2).sum(-1, keepdim=True) + 1e-6) * dk ** -0.5
+        k = x["k"] / torch.sqrt((x["k"] ** 2).sum(-1, keepdim=True) + 1e-6)
+        beta = torch.sigmoid(x["b"])
+        gate = torch.exp(-torch.exp(A_log.double()) * torch.nn.functional.softplus(x["a"] + dt_bias.double()))
+        want = O.delta_rule(q.repeat_interleave(H // G, 1), k.repeat_interleave(H // G, 1), x["v"], beta, gate)
+        assert row_err(torch.cat(got[i]), want.reshape(T, -1)) < 1e-5
+
+
+def _attention_case(dt, H, G, d, dv, size, keep, past, n_new, hot):
+    """One sequence with ``past`` cached keys and ``n_new`` queries.  Every key is small noise except the ``hot`` ones, which match the query direction
+    with a large score and carry a marked value: whether a query's output shows the mark says whether it saw the key."""
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(size * 131 + past)
+    T = past + n_new
+    qdir = torch.randn(d, generator=g)
+    qdir = qdir / qdir.norm()
+    q = qdir.repeat(T, H, 1) * 6 + 0.1 * torch.randn(T, H, d, generator=g)
+    k = 0.1 * torch.randn(T, G, d, generator=g)
+    v = torch.randn(T, G, dv, generator=g)
+    for j in hot:
+        k[j] = qdir * 6
+        v[j] = 100.0
+    temp = torch.rand(H, generator=g) + 0.5
+    cdt = F32 if dt == "float32" else BF16
+    kq, vq = k.to(cdt), v.to(cdt)
+    want = O.window_attention(q.double(), kq.double(), vq.double(), 0.3, temp.double(), size, keep, first_query=past)[past:]
+    cache = torch.zeros(T + 5, G * (d + dv), dtype=cdt, device=DEV)
+    cache[:T, : G * d] = kq.reshape(T, -1).to(DEV)
+    cache[:T, G * d :] = vq.reshape(T, -1).to(DEV)
+    qs = (q[past:] * (0.3 * temp)[None, :, None]).reshape(n_new, H * d).to(DEV).contiguous()
+    out = torch.empty(n_new, H * dv, dtype=cdt, device=DEV)
+    hm = 1
+    while hm * 2 <= 32 and (H // G) % (hm * 2) == 0:
+        hm *= 2
+    desc = (dev_i32([0]), dev_i32([n_new]), dev_i32([past]), dev_i32([0]), dev_i32([0]), dev_i32([0]))
+    S.latent_attn(qs, cache, None, cache[:, G * d :], out, H, hm, d, 0, dv, d, d, dv, dv, desc, n_new, 1.0, max_keys=T, kv_rep=H // G, window=size, keep_first=keep)
+    return out.float().cpu().reshape(n_new, H, dv), want
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,d,dv", [(4, 2, 24, 40), (6, 2, 64, 64), (3, 3, 136, 16)])
+def test_attention_window_and_kept_tokens_edges_in_prompts(dt, H, G, d, dv):
+    """Hot keys at the last kept position and the first one not kept, and at positions that are just inside / just outside the window of chosen queries,
+    also across the kernels' 64-key and 128-query steps."""
+    size, keep, T = 70, 5, 300
+    hot = [keep - 1, keep, 100, 200 - size, 200 - size + 1]
+    got, want = _attention_case(dt, H, G, d, dv, size, keep, 0, T, hot)
+    assert row_err(got.reshape(T, -1), want.reshape(T, -1)) < (2e-5 if dt == "float32" else 2e-2)
+    w = want[:, 0, 0]
+    assert abs(w[2]) < 10 and w[keep - 1] > 30 and w[299] > 30  # the oracle itself: the last kept token marks every later query
+    far = _attention_case(dt, H, G, d, dv, size, 0, 0, T, [100])
+    assert far[1][100 + size - 1, 0, 0] > 30 and abs(far[1][100 + size, 0, 0]) < 10  # the oracle itself: inside, then outside
+    assert row_err(far[0].reshape(T, -1), far[1].reshape(T, -1)) < (2e-5 if dt == "float32" else 2e-2)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_new", [1, 3])
+def test_attention_window_and_kept_tokens_edges_in_decoding(dt, n_new):
+    size, keep = 70, 5
+    for past in (63, 64, 69, 70, 71, 127, 128, 129, 400):
+        last = past + n_new - 1
+        for hot in ([last - size + 1], [last - size], [keep - 1], [keep], [last]):
+            hot = [j for j in hot if 0 <= j <= last]
+            if not hot:
+                continue
+            got, want = _attention_case(dt, 6, 3, 32, 48, size, keep, past, n_new, hot)
+            assert row_err(got.reshape(n_new, -1), want.reshape(n_new, -1)) < (2e-5 if dt == "float32" else 2e-2), (past, hot)
+
+
+def test_query_key_value_rows():
+    """Bias, head norm, partial interleaved rotation, per-head query scale; keys and values land in the cache rows they are sent to."""
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(4)
+    T, H, G, d, dv, dims = 5, 3, 1, 20, 12, 8
+    n = (H + G) * d + G * dv
+    src, bias = torch.randn(T, n, generator=g), torch.randn(n, generator=g)
+    qw, kw, qs = torch.rand(d, generator=g) + 0.5, torch.rand(d, generator=g) + 0.5, torch.rand(H, generator=g) + 0.5
+    pos, rows = [0, 1, 70, 1000, 5], [9, 2, 0, 7, 4]
+    cache = torch.zeros(10, G * (d + dv), device=DEV)
+    q = S.qkv_rows_append(src.to(DEV), H, G, d, dv, bias.to(DEV), qw.to(DEV), kw.to(DEV), 1e-6, qs.to(DEV), dims, 0, S.rope_frequencies(dims, 500.0, DEV), dev_i32(pos), dev_i32(rows), cache)
+    x = (src + bias).double()
+    full = torch.zeros(1001, H + G, d, dtype=F64)
+    heads = x[:, : (H + G) * d].reshape(T, H + G, d)
+    normed = O.unit_rms(heads, 1e-6) * torch.cat([qw.double().repeat(H, 1), kw.double().repeat(G, 1)])[None]
+    full[pos] = normed
+    rot = O.rotary(full, dims, 500.0, "interleaved")[pos]
+    assert row_err(q, (rot[:, :H] * qs.double()[None, :, None]).reshape(T, -1)) < 1e-5
+    assert row_err(cache[rows, : G * d], rot[:, H:].reshape(T, -1)) < 1e-5
+    assert torch.allclose(cache[rows, G * d :].cpu().double(), x[:, (H + G) * d :], atol=1e-6)
+
+
+def test_softmax_router_and_gated_activations():
+    from llm_quest_amd import kernels_seq as S
+
+    g = torch.Generator().manual_seed(5)
+    for E, top in ((5, 1), (16, 2), (70, 6), (200, 3)):
+        logits = torch.randn(33, E, generator=g) * 3
+        ids, wts = S.moe_route(logits.to(DEV), None, top, 1, 1, 1.0, softmax=True)
+        s = torch.softmax(logits.double(), -1)
+        wv, wi = torch.topk(s, top, -1)
+        assert torch.equal(ids.cpu().long(), wi) and torch.allclose(wts.cpu().double(), wv, rtol=1e-5, atol=1e-7)
+    x = torch.randn(7, 2 * 37, generator=g) * 3
+    gate, up = x[:, :37].double(), x[:, 37:].double()
+    assert row_err(S.glu_rows(x.to(DEV), S.GLU_GELU_TANH), O.gelu_tanh(gate) * up) < 1e-6
+    gc, uc = gate.clamp(max=1.5), up.clamp(-1.5, 1.5)
+    assert row_err(S.glu_rows(x.to(DEV), S.GLU_CLAMPED_SWISH, 1.5), gc * torch.sigmoid(1.702 * gc) * (uc + 1)) < 1e-6
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_mixture_of_experts_alone(dt):
+    from llm_quest_amd.common.mixers import SoftmaxTopkMoE
+
+    g = torch.Generator().manual_seed(6)
+    W, ff, E, top, T = 72, 40, 11, 3, 50
+    cfg = U.make_config([(U.retention(), U.moe(experts=E, top=top, ff=ff, limit=0.8))], width=W)
+    w = U.make_weights(cfg, 3)
+    m = SoftmaxTopkMoE(W, ff, E, top, 0.8)
+    m.w_router.data.copy_(w["l0.mlp.router"])
+    m.w_gate_up.data.copy_(torch.stack([torch.cat([w[f"l0.mlp.e{j}.gate"], w[f"l0.mlp.e{j}.up"]]) for j in range(E)]))
+    m.w_down.data.copy_(torch.stack([w[f"l0.mlp.e{j}.down"] for j in range(E)]))
+    m = m.to(DEV)
+    h = torch.randn(T, W, generator=g)
+    act = F32 if dt == "float32" else BF16
+    hq = h.to(act)
+    out = m.step(h.to(DEV), hq.to(DEV)).reshape(T, top, W).sum(1)
+    wd = {k: v.double() for k, v in w.items()}
+    ids, wts = O.route(h.double(), wd["l0.mlp.router"], top)
+    want = torch.zeros(T, W, dtype=F64)
+    for t in range(T):
+        for e, a in zip(ids[t].tolist(), wts[t]):
+            want[t] += a * O.expert_ff(hq[t : t + 1].double(), wd, f"l0.mlp.e{e}.", 0.8)[0]
+    assert row_err(out, want) < (1e-5 if dt == "float32" else 2e-2)
