@@ -588,10 +588,10 @@ int mi355_qkv_rows_append(int64_t tokens, int H, int G, int d, int dv, const voi
 /* Gated delta rule over the rows [seq_off[s], seq_off[s+1]) of each sequence, state[slot[s]] (fp32 [H, dk, dv]) read and written.  q / k rows [G * dk] (raw:
  * made unit vectors here, x / sqrt(sum x^2 + 1e-6), q also times qscale), v rows [H * dv]; value head h uses query / key head h / (H / G);
  * beta = sigmoid(b[t, h]), g = exp(-exp(A_log[h]) * softplus(a[t, h] + dt_bias[h])).  Per token: S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
- * o fp32 [tokens, H * dv].  dk <= 256. */
-int mi355_delta_rule_ragged(int n_seq, const int* seq_off, const int* slot, int H, int G, int dk, int dv, const void* q, const void* k, int qk_dt, int64_t ldq,
-                            int64_t ldk, const void* v, int v_dt, int64_t ldv, const void* b, const void* a, int ba_dt, int64_t ldb, int64_t lda,
-                            const float* A_log, const float* dt_bias, float qscale, float* state, float* o, void* stream);
+ * o fp32 [tokens, H * dv].  dk <= 256.  `tokens` = all rows of the step; ws: 16-byte aligned scratch of tokens * H * 4 floats (the per-token scalars). */
+int mi355_delta_rule_ragged(int64_t tokens, int n_seq, const int* seq_off, const int* slot, int H, int G, int dk, int dv, const void* q, const void* k, int qk_dt,
+                            int64_t ldq, int64_t ldk, const void* v, int v_dt, int64_t ldv, const void* b, const void* a, int ba_dt, int64_t ldb, int64_t lda,
+                            const float* A_log, const float* dt_bias, float qscale, float* state, float* o, float* ws, void* stream);
 /* Gated feed-forward activation on rows [gate (F) | up (F)] -> [F].  kind 0: gelu_tanh(gate) * up.  kind 1: g = min(gate, limit), u = clamp(up, -limit, limit),
  * g * sigmoid(1.702 g) * (u + 1). */
 int mi355_glu_rows(int64_t rows, int F, const void* in, int in_dt, int64_t ld_in, int kind, float limit, void* out, int out_dt, int64_t ld_out, void* stream);

@@ -117,7 +117,7 @@ SIGNATURES = {
     "mi355_group_rmsnorm_sum": [_L, _I, _P, _P, _I, _L, _P, _I, _L, _I, _P, _I, _F, _P, _P, _I, _P, _P, _P, _I, _P, _P],
     "mi355_ragged_conv": [_L, _I, _I, _I, _P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _P, _I, _L, _P],
     "mi355_qkv_rows_append": [_L, _I, _I, _I, _I, _P, _I, _L, _P, _P, _P, _F, _P, _I, _I, _P, _P, _P, _P, _L, _P, _I, _L, _P],
-    "mi355_delta_rule_ragged": [_I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _L, _L, _P, _I, _L, _P, _P, _I, _L, _L, _P, _P, _F, _P, _P, _P],
+    "mi355_delta_rule_ragged": [_L, _I, _P, _P, _I, _I, _I, _I, _P, _P, _I, _L, _L, _P, _I, _L, _P, _P, _I, _L, _L, _P, _P, _F, _P, _P, _P, _P],
     "mi355_glu_rows": [_L, _I, _P, _I, _L, _I, _F, _P, _I, _L, _P],
     # measurement aid (csrc/probe.hip)
     "mi355_mfma_pipe_probe": [_I, _I, _P, _P],

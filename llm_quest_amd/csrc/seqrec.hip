@@ -19,6 +19,17 @@ static inline int rec_rows_grid(int64_t rows, int per_block) {
     return (int)(g < 1 ? 1 : (g > 65535 * 16 ? 65535 * 16 : g));
 }
 static inline bool rec_dt_ok(int dt) { return dt == MI355_DT_BF16 || dt == MI355_DT_F32; }
+// four consecutive elements (the caller vouches for 16-byte alignment of fp32 rows, 8-byte of bf16 rows)
+__device__ __forceinline__ f32x4 ld4_dt(const void* p, int dt, int64_t i) {
+    if (dt == MI355_DT_F32) return *(const f32x4*)((const float*)p + i);
+    const u32x2 r = *(const u32x2*)((const bf16_t*)p + i);
+    return f32x4{__uint_as_float(r[0] << 16), __uint_as_float(r[0] & 0xffff0000u), __uint_as_float(r[1] << 16), __uint_as_float(r[1] & 0xffff0000u)};
+}
+__device__ __forceinline__ void st4_dt(void* p, int dt, int64_t i, f32x4 v) {
+    if (dt == MI355_DT_F32) *(f32x4*)((float*)p + i) = v;
+    else *(u32x2*)((bf16_t*)p + i) = u32x2{pack_bf2(v[0], v[1]), pack_bf2(v[2], v[3])};
+}
+static inline bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 // ------------------------------------------------------------------------------------------- residual sum + RMS norms in groups
 // v = x + y1[t] + sum_{p < parts} y2[t * parts + p]  (fp32; either summand may be absent); x_out (optional, may be x) receives v.
@@ -94,6 +105,65 @@ __global__ __launch_bounds__(256) void group_rmsnorm_sum_kernel(int64_t T, int w
     }
 }
 
+// The same for wide rows: one workgroup per row, 16-byte accesses; thread t owns elements 4 (t + 256 j) .. + 4 (a group's size is a multiple of 4, so
+// the four lie in one group).  A wave sums its share of every group, the four waves' shares meet in LDS in a fixed order.
+#define GN_MAXG 64
+template <int V4>
+__global__ __launch_bounds__(256) void group_rmsnorm_sum_wide_kernel(int64_t T, int width, GroupNormArgs p) {
+    __shared__ float red[4][GN_MAXG];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int gs = width / p.groups;
+    for (int64_t t = blockIdx.x; t < T; t += gridDim.x) {
+        f32x4 v[V4];
+        int grp[V4];
+#pragma unroll
+        for (int j = 0; j < V4; ++j) {
+            const int i = 4 * (tid + 256 * j);
+            f32x4 a = {0.f, 0.f, 0.f, 0.f};
+            grp[j] = -1;
+            if (i < width) {
+                grp[j] = i / gs;
+                a = *(const f32x4*)(p.x + t * width + i);
+                f32x4 ys = {0.f, 0.f, 0.f, 0.f};
+                if (p.y1) ys = ld4_dt(p.y1, p.y1_dt, t * p.ldy1 + i);
+                if (p.y2) {
+                    f32x4 y2s = {0.f, 0.f, 0.f, 0.f};
+                    for (int q = 0; q < p.parts; ++q) y2s += ld4_dt(p.y2, p.y2_dt, (t * p.parts + q) * p.ldy2 + i);
+                    ys += y2s;
+                }
+                a += ys;
+                if (p.x_out) *(f32x4*)(p.x_out + t * width + i) = a;
+            }
+            v[j] = a;
+        }
+        if (!p.w[0] && !p.w[1]) continue;
+        for (int g = 0; g < p.groups; ++g) {
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < V4; ++j)
+                if (grp[j] == g) s += (v[j][0] * v[j][0] + v[j][1] * v[j][1]) + (v[j][2] * v[j][2] + v[j][3] * v[j][3]);
+            s = wave_sum(s);
+            if (lane == 0) red[wave][g] = s;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < V4; ++j) {
+            const int i = 4 * (tid + 256 * j);
+            if (i >= width) continue;
+            const int g = grp[j];
+            const float r = 1.0f / sqrtf(((red[0][g] + red[1][g]) + (red[2][g] + red[3][g])) / (float)gs + p.eps);
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
+                if (!p.w[n]) continue;
+                const f32x4 o = v[j] * r * *(const f32x4*)(p.w[n] + i);
+                if (p.out[n]) st4_dt(p.out[n], p.out_dt[n], t * width + i, o);
+                if (p.out32[n]) *(f32x4*)(p.out32[n] + t * width + i) = o;
+            }
+        }
+        __syncthreads();  // red[] is reused by the next row
+    }
+}
+
 extern "C" int mi355_group_rmsnorm_sum(int64_t tokens, int width, const float* x, const void* y1, int y1_dt, int64_t ldy1, const void* y2, int y2_dt, int64_t ldy2,
                                        int parts, float* x_out, int groups, float eps, const float* w_a, void* out_a, int out_a_dt, float* out_a32, const float* w_b,
                                        void* out_b, int out_b_dt, float* out_b32, void* stream) {
@@ -107,6 +177,19 @@ extern "C" int mi355_group_rmsnorm_sum(int64_t tokens, int width, const float* x
     p.w[0] = w_a, p.w[1] = w_b, p.out[0] = out_a, p.out[1] = out_b, p.out32[0] = out_a32, p.out32[1] = out_b32;
     p.ldy1 = ldy1, p.ldy2 = ldy2, p.y1_dt = y1_dt, p.y2_dt = y2_dt, p.parts = parts, p.groups = groups, p.out_dt[0] = out_a_dt, p.out_dt[1] = out_b_dt;
     p.eps = eps;
+    const bool wide = width > 256 && width % 4 == 0 && (width / groups) % 4 == 0 && groups <= GN_MAXG && al16(x) && (!y1 || (al16(y1) && ldy1 % 4 == 0)) &&
+                      (!y2 || (al16(y2) && ldy2 % 4 == 0)) && al16(x_out) && al16(w_a) && al16(w_b) && al16(out_a) && al16(out_b) && al16(out_a32) && al16(out_b32);
+    if (wide) {
+        const int g = (int)(tokens < 65535 * 8 ? tokens : 65535 * 8);
+#define GNW_CASE(V)                                                                         \
+    if (width <= 1024 * V) {                                                                \
+        group_rmsnorm_sum_wide_kernel<V><<<g, 256, 0, ST(stream)>>>(tokens, width, p);      \
+        MI355_LAUNCH_CHECK("group_rmsnorm_sum");                                            \
+        return 0;                                                                           \
+    }
+        GNW_CASE(1) GNW_CASE(2) GNW_CASE(4) GNW_CASE(8)
+#undef GNW_CASE
+    }
     const int grid = rec_rows_grid(tokens, 4);
 #define GN_CASE(E)                                                                      \
     if (width <= 64 * E) {                                                              \
@@ -147,6 +230,33 @@ __global__ __launch_bounds__(256) void ragged_conv_kernel(int64_t T, int C, int 
     }
 }
 
+// Four channels per thread, one token per blockIdx.x (C % 4 == 0, 16-byte aligned rows).
+__global__ __launch_bounds__(256) void ragged_conv_vec_kernel(int C, int taps, const void* __restrict__ x, int x_dt, int64_t ldx, const float* __restrict__ w,
+                                                              const int* __restrict__ row_seq, const int* __restrict__ seq_off, const int* __restrict__ slot,
+                                                              const float* __restrict__ state, int act, int residual, void* __restrict__ y, int y_dt, int64_t ldy) {
+    const int64_t t = blockIdx.x;
+    const int c = 4 * (blockIdx.y * 256 + threadIdx.x);
+    if (c >= C) return;
+    const int s = row_seq[t];
+    const int start = seq_off[s];
+    const int local = (int)(t - start);
+    const float* st = state + (int64_t)slot[s] * (taps - 1) * C;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f}, cur = {0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < taps; ++j) {
+        const int sl = local - (taps - 1) + j;
+        const f32x4 in = sl >= 0 ? ld4_dt(x, x_dt, (int64_t)(start + sl) * ldx + c) : *(const f32x4*)(st + (int64_t)(taps - 1 + sl) * C + c);
+        if (j == taps - 1) cur = in;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = fmaf(w[(c + e) * taps + j], in[e], acc[e]);
+    }
+    if (act == 1) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = acc[e] / (1.0f + expf(-acc[e]));
+    }
+    if (residual) acc += cur;
+    st4_dt(y, y_dt, t * ldy + c, acc);
+}
+
 __global__ __launch_bounds__(256) void ragged_conv_state_kernel(int n_seq, int C, int taps, const void* __restrict__ x, int x_dt, int64_t ldx, const int* __restrict__ seq_off,
                                                                 const int* __restrict__ slot, float* __restrict__ state) {
     const int64_t total = (int64_t)n_seq * C;
@@ -175,8 +285,12 @@ extern "C" int mi355_ragged_conv(int64_t tokens, int n_seq, int C, int taps, con
                   "ragged_conv: bad arguments (taps <= 16)");
     MI355_REQUIRE(rec_dt_ok(x_dt) && rec_dt_ok(y_dt) && ldx >= C && ldy >= C && (act == 0 || act == 1), "ragged_conv: bad operands");
     const int64_t total = tokens * C;
-    const int g = (int)((total + 255) / 256 > 65535 * 8 ? 65535 * 8 : (total + 255) / 256);
-    ragged_conv_kernel<<<g, 256, 0, ST(stream)>>>(tokens, C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy);
+    if (C % 4 == 0 && ldx % 4 == 0 && ldy % 4 == 0 && al16(x) && al16(y) && al16(state) && tokens < ((int64_t)1 << 31)) {
+        ragged_conv_vec_kernel<<<dim3((unsigned)tokens, (C / 4 + 255) / 256), 256, 0, ST(stream)>>>(C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy);
+    } else {
+        const int g = (int)((total + 255) / 256 > 65535 * 8 ? 65535 * 8 : (total + 255) / 256);
+        ragged_conv_kernel<<<g, 256, 0, ST(stream)>>>(tokens, C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy);
+    }
     MI355_LAUNCH_CHECK("ragged_conv");
     if (taps > 1) {
         const int64_t tot2 = (int64_t)n_seq * C;
@@ -268,130 +382,152 @@ extern "C" int mi355_qkv_rows_append(int64_t tokens, int H, int G, int d, int dv
 //   k^ = k / sqrt(sum k^2 + 1e-6), q^ = q / sqrt(sum q^2 + 1e-6) * qscale   (unit vectors; raw q / k rows come in)
 //   beta = sigmoid(b), g = exp(-exp(A_log[h]) * softplus(a + dt_bias[h]))
 //   S <- g S;  u = beta (v - S^T k^);  S <- S + k^ u^T;  o = S^T q^
-// Block: 64 value columns x RC chunks of DR_R key channels; a thread keeps DR_R state entries of one column in registers.  The unit-vector factors are
-// scalars per token, so the raw rows are staged and the factors applied to the column's dot products.  Tokens go through in groups of DR_TB; within a
-// group one barrier per token lets the chunks' partial S^T k meet (none when one chunk holds all key channels).
-#define DR_R 32
-#define DR_TB 8
+// Column c of S obeys its own recurrence, so columns are spread over lanes and the time loop stays inside: DR_LPR lanes share a column (CPL key
+// channels each, in registers), the two dot products of a step close with lane sums -- no LDS, no barrier.  The per-token scalars (g, beta and the two
+// unit-vector factors, which multiply the dot products instead of the rows) are prepared once per (token, head) by delta_prep_kernel; the operands of
+// step t + 1 are requested before step t's arithmetic.
+#define DR_LPR 8
 struct DeltaArgs {
     const int *seq_off, *slot;
     const void *q, *k, *v, *b, *a;
     const float *A_log, *dt_bias;
     float *state, *o;
+    f32x4* ws;  // [tokens, H]: g, beta, key factor, query factor * qscale
     int64_t ldq, ldk, ldv, ldb, lda;
     int H, G, dk, dv, qk_dt, v_dt, ba_dt;
     float qscale;
 };
 
-__global__ __launch_bounds__(512) void delta_rule_kernel(DeltaArgs p) {
-    extern __shared__ __attribute__((aligned(16))) float smem[];
-    const int RC = blockDim.x >> 6, dk = p.dk;
-    float* sq = smem;                       // [TB][dk]
-    float* sk = sq + DR_TB * dk;            // [TB][dk]
-    float* sv = sk + DR_TB * dk;            // [TB][64]
-    float* sc = sv + DR_TB * 64;            // [TB][4]: beta, g, key factor, query factor
-    float* sp = sc + DR_TB * 4;             // [2][RC][64]
-    float* so = sp + 2 * RC * 64;           // [TB][RC][64]
-    const int s = blockIdx.x, h = blockIdx.y, lc = threadIdx.x & 63, col = blockIdx.z * 64 + lc, chunk = threadIdx.x >> 6, lane = lc;
-    const int hq = h / (p.H / p.G);
-    const int t0 = p.seq_off[s], t1 = p.seq_off[s + 1];
-    const bool col_ok = col < p.dv;
-    float* S = p.state + (((int64_t)p.slot[s] * p.H + h) * dk) * p.dv;
-    float st[DR_R];
-#pragma unroll
-    for (int r = 0; r < DR_R; ++r) {
-        const int i = chunk * DR_R + r;
-        st[r] = (col_ok && i < dk) ? S[(int64_t)i * p.dv + col] : 0.f;
-    }
-    const float neg_A = -expf(p.A_log[h]), dtb = p.dt_bias[h];
-    for (int tb = t0; tb < t1; tb += DR_TB) {
-        const int nt = min(DR_TB, t1 - tb);
-        __syncthreads();
-        for (int e = threadIdx.x; e < nt * dk; e += blockDim.x) {
-            const int j = e / dk, i = e % dk;
-            sq[e] = ldr_dt(p.q, p.qk_dt, (int64_t)(tb + j) * p.ldq + (int64_t)hq * dk + i);
-            sk[e] = ldr_dt(p.k, p.qk_dt, (int64_t)(tb + j) * p.ldk + (int64_t)hq * dk + i);
+__global__ __launch_bounds__(256) void delta_prep_kernel(int64_t T, DeltaArgs p) {
+    const int lane = threadIdx.x & 63;
+    const int64_t items = T * p.H;
+    for (int64_t it = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); it < items; it += (int64_t)gridDim.x * 4) {
+        const int64_t t = it / p.H;
+        const int h = (int)(it % p.H), hq = h / (p.H / p.G);
+        float sq = 0.f, sk = 0.f;
+        for (int i = lane; i < p.dk; i += 64) {
+            const float qv = ldr_dt(p.q, p.qk_dt, t * p.ldq + (int64_t)hq * p.dk + i), kv = ldr_dt(p.k, p.qk_dt, t * p.ldk + (int64_t)hq * p.dk + i);
+            sq += qv * qv;
+            sk += kv * kv;
         }
-        for (int e = threadIdx.x; e < nt * 64; e += blockDim.x) {
-            const int j = e >> 6, c = blockIdx.z * 64 + (e & 63);
-            sv[e] = c < p.dv ? ldr_dt(p.v, p.v_dt, (int64_t)(tb + j) * p.ldv + (int64_t)h * p.dv + c) : 0.f;
+        sq = wave_sum(sq);
+        sk = wave_sum(sk);
+        if (lane == 0) {
+            const float bb = ldr_dt(p.b, p.ba_dt, t * p.ldb + h), aa = ldr_dt(p.a, p.ba_dt, t * p.lda + h) + p.dt_bias[h];
+            const float sp = aa > 20.f ? aa : log1pf(expf(aa));
+            p.ws[it] = f32x4{expf(-expf(p.A_log[h]) * sp), 1.0f / (1.0f + expf(-bb)), 1.0f / sqrtf(sk + 1e-6f), p.qscale / sqrtf(sq + 1e-6f)};
         }
-        if (threadIdx.x < nt) {
-            const int j = threadIdx.x;
-            const float bb = ldr_dt(p.b, p.ba_dt, (int64_t)(tb + j) * p.ldb + h), aa = ldr_dt(p.a, p.ba_dt, (int64_t)(tb + j) * p.lda + h) + dtb;
-            const float sp_ = aa > 20.f ? aa : log1pf(expf(aa));
-            sc[4 * j + 0] = 1.0f / (1.0f + expf(-bb));
-            sc[4 * j + 1] = expf(neg_A * sp_);
-        }
-        __syncthreads();
-        // unit-vector factors: item (token j, q or k) per wave, round-robin
-        for (int it = chunk; it < 2 * nt; it += RC) {
-            const int j = it >> 1;
-            const float* row = (it & 1) ? sq + j * dk : sk + j * dk;
-            float ss = 0.f;
-            for (int i = lane; i < dk; i += 64) ss += row[i] * row[i];
-            ss = wave_sum(ss);
-            if (lane == 0) sc[4 * j + 2 + (it & 1)] = (1.0f / sqrtf(ss + 1e-6f)) * ((it & 1) ? p.qscale : 1.0f);
-        }
-        __syncthreads();
-        for (int j = 0; j < nt; ++j) {
-            const float* ka = sk + j * dk + chunk * DR_R;
-            const float* qa = sq + j * dk + chunk * DR_R;
-            const float beta = sc[4 * j], g = sc[4 * j + 1], kn = sc[4 * j + 2];
-            float part = 0.f;
-#pragma unroll
-            for (int r = 0; r < DR_R; ++r)
-                if (chunk * DR_R + r < dk) part += st[r] * ka[r];
-            float Sk = part;
-            if (RC > 1) {
-                float* buf = sp + (j & 1) * RC * 64;
-                buf[chunk * 64 + lc] = part;
-                __syncthreads();
-                Sk = 0.f;
-                for (int rc = 0; rc < RC; ++rc) Sk += buf[rc * 64 + lc];
-            }
-            const float u = beta * (sv[j * 64 + lc] - g * kn * Sk);
-            const float uk = u * kn;
-            float acc = 0.f;
-#pragma unroll
-            for (int r = 0; r < DR_R; ++r)
-                if (chunk * DR_R + r < dk) {
-                    st[r] = g * st[r] + ka[r] * uk;
-                    acc += st[r] * qa[r];
-                }
-            so[(j * RC + chunk) * 64 + lc] = acc;
-        }
-        __syncthreads();
-        for (int e = threadIdx.x; e < nt * 64; e += blockDim.x) {
-            const int j = e >> 6, c = blockIdx.z * 64 + (e & 63);
-            if (c < p.dv) {
-                float acc = 0.f;
-                for (int rc = 0; rc < RC; ++rc) acc += so[(j * RC + rc) * 64 + (e & 63)];
-                p.o[(int64_t)(tb + j) * p.H * p.dv + (int64_t)h * p.dv + c] = acc * sc[4 * j + 3];
-            }
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < DR_R; ++r) {
-        const int i = chunk * DR_R + r;
-        if (col_ok && i < dk) S[(int64_t)i * p.dv + col] = st[r];
     }
 }
 
-extern "C" int mi355_delta_rule_ragged(int n_seq, const int* seq_off, const int* slot, int H, int G, int dk, int dv, const void* q, const void* k, int qk_dt, int64_t ldq,
-                                       int64_t ldk, const void* v, int v_dt, int64_t ldv, const void* b, const void* a, int ba_dt, int64_t ldb, int64_t lda,
-                                       const float* A_log, const float* dt_bias, float qscale, float* state, float* o, void* stream) {
-    MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && seq_off && slot && H > 0 && H <= 65535 && G > 0 && H % G == 0 && dk > 0 && dk <= 8 * DR_R && dv > 0 && q && k && v && b && a &&
-                      A_log && dt_bias && state && o,
-                  "delta_rule_ragged: bad arguments (key channels per head <= 256, value heads a multiple of the query / key heads)");
+template <int CPL, bool VEC>
+__global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs p) {
+    constexpr int RPW = 64 / DR_LPR;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int s = blockIdx.z, h = blockIdx.y;
+    const int col0 = (blockIdx.x * 4 + wave) * RPW;
+    if (col0 >= p.dv) return;  // whole wave out of range; no block-level synchronisation below
+    const int col = col0 + lane / DR_LPR, cg = lane % DR_LPR, ch0 = cg * CPL;
+    const bool col_ok = col < p.dv;
+    const int hq = h / (p.H / p.G), dk = p.dk;
+    const int t0 = p.seq_off[s], t1 = p.seq_off[s + 1];
+    float* S = p.state + (((int64_t)p.slot[s] * p.H + h) * dk) * p.dv;
+    float st[CPL];
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) st[i] = (col_ok && ch0 + i < dk) ? S[(int64_t)(ch0 + i) * p.dv + col] : 0.f;
+    struct In {
+        float k[CPL], q[CPL];
+        f32x4 sc;
+        float v;
+    };
+    auto load_in = [&](In& in, int t) {
+        const int64_t ko = (int64_t)t * p.ldk + (int64_t)hq * dk + ch0, qo = (int64_t)t * p.ldq + (int64_t)hq * dk + ch0;
+        if (VEC) {
+#pragma unroll
+            for (int i = 0; i < CPL; i += 4) {
+                f32x4 kv = {0.f, 0.f, 0.f, 0.f}, qv = {0.f, 0.f, 0.f, 0.f};
+                if (ch0 + i < dk) {
+                    kv = *(const f32x4*)((const float*)p.k + ko + i);
+                    qv = *(const f32x4*)((const float*)p.q + qo + i);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) in.k[i + e] = kv[e], in.q[i + e] = qv[e];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < CPL; ++i) {
+                const bool ok = ch0 + i < dk;
+                in.k[i] = ok ? ldr_dt(p.k, p.qk_dt, ko + i) : 0.f;
+                in.q[i] = ok ? ldr_dt(p.q, p.qk_dt, qo + i) : 0.f;
+            }
+        }
+        in.sc = p.ws[(int64_t)t * p.H + h];
+        in.v = col_ok ? ldr_dt(p.v, p.v_dt, (int64_t)t * p.ldv + (int64_t)h * p.dv + col) : 0.f;
+    };
+    auto step = [&](const In& in, int t) {
+        const float a = in.sc[0], b = in.sc[1], kn = in.sc[2], qn = in.sc[3];
+        float u0 = 0.f, u1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < CPL; i += 2) {
+            st[i] *= a;
+            st[i + 1] *= a;
+            u0 = fmaf(st[i], in.k[i], u0);
+            u1 = fmaf(st[i + 1], in.k[i + 1], u1);
+        }
+        const float u = lanes_sum<DR_LPR>(u0 + u1) * kn;
+        const float c = b * (in.v - u) * kn;
+        float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < CPL; i += 2) {
+            st[i] = fmaf(c, in.k[i], st[i]);
+            st[i + 1] = fmaf(c, in.k[i + 1], st[i + 1]);
+            o0 = fmaf(st[i], in.q[i], o0);
+            o1 = fmaf(st[i + 1], in.q[i + 1], o1);
+        }
+        const float oo = lanes_sum<DR_LPR>(o0 + o1) * qn;
+        if (cg == 0 && col_ok) p.o[(int64_t)t * p.H * p.dv + (int64_t)h * p.dv + col] = oo;
+    };
+    In inA, inB;
+    if (t0 < t1) load_in(inA, t0);
+    for (int t = t0; t < t1; t += 2) {
+        if (t + 1 < t1) load_in(inB, t + 1);
+        step(inA, t);
+        if (t + 1 < t1) {
+            if (t + 2 < t1) load_in(inA, t + 2);
+            step(inB, t + 1);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < CPL; ++i)
+        if (col_ok && ch0 + i < dk) S[(int64_t)(ch0 + i) * p.dv + col] = st[i];
+}
+
+template <int CPL>
+static void launch_delta(const DeltaArgs& p, dim3 grid, bool vec, hipStream_t st) {
+    if (vec) delta_rule_kernel<CPL, true><<<grid, 256, 0, st>>>(p);
+    else delta_rule_kernel<CPL, false><<<grid, 256, 0, st>>>(p);
+}
+
+extern "C" int mi355_delta_rule_ragged(int64_t tokens, int n_seq, const int* seq_off, const int* slot, int H, int G, int dk, int dv, const void* q, const void* k, int qk_dt,
+                                       int64_t ldq, int64_t ldk, const void* v, int v_dt, int64_t ldv, const void* b, const void* a, int ba_dt, int64_t ldb, int64_t lda,
+                                       const float* A_log, const float* dt_bias, float qscale, float* state, float* o, float* ws, void* stream) {
+    MI355_REQUIRE(tokens > 0 && n_seq > 0 && n_seq <= 65535 && seq_off && slot && H > 0 && H <= 65535 && G > 0 && H % G == 0 && dk > 0 && dk <= 32 * DR_LPR && dv > 0 && q && k && v &&
+                      b && a && A_log && dt_bias && state && o && ws,
+                  "delta_rule_ragged: bad arguments (key channels per head <= 256, value heads a multiple of the query / key heads, workspace of 4 floats per token and head)");
     MI355_REQUIRE(rec_dt_ok(qk_dt) && rec_dt_ok(v_dt) && rec_dt_ok(ba_dt) && ldq >= (int64_t)G * dk && ldk >= (int64_t)G * dk && ldv >= (int64_t)H * dv && ldb >= H && lda >= H,
                   "delta_rule_ragged: rows too short");
+    MI355_REQUIRE(((uintptr_t)ws & 15) == 0, "delta_rule_ragged: the workspace must be 16-byte aligned");
     DeltaArgs p;
-    p.seq_off = seq_off, p.slot = slot, p.q = q, p.k = k, p.v = v, p.b = b, p.a = a, p.A_log = A_log, p.dt_bias = dt_bias, p.state = state, p.o = o;
+    p.seq_off = seq_off, p.slot = slot, p.q = q, p.k = k, p.v = v, p.b = b, p.a = a, p.A_log = A_log, p.dt_bias = dt_bias, p.state = state, p.o = o, p.ws = (f32x4*)ws;
     p.ldq = ldq, p.ldk = ldk, p.ldv = ldv, p.ldb = ldb, p.lda = lda, p.H = H, p.G = G, p.dk = dk, p.dv = dv, p.qk_dt = qk_dt, p.v_dt = v_dt, p.ba_dt = ba_dt, p.qscale = qscale;
-    const int RC = (dk + DR_R - 1) / DR_R;
-    const size_t lds_bytes = sizeof(float) * ((size_t)2 * DR_TB * dk + (size_t)DR_TB * 64 + DR_TB * 4 + (size_t)2 * RC * 64 + (size_t)DR_TB * RC * 64);
-    delta_rule_kernel<<<dim3(n_seq, H, (dv + 63) / 64), 64 * RC, lds_bytes, ST(stream)>>>(p);
+    delta_prep_kernel<<<rec_rows_grid(tokens * H, 4), 256, 0, ST(stream)>>>(tokens, p);
+    MI355_LAUNCH_CHECK("delta_rule_ragged(prep)");
+    const bool vec = qk_dt == MI355_DT_F32 && dk % 4 == 0 && ldq % 4 == 0 && ldk % 4 == 0 && ((uintptr_t)q & 15) == 0 && ((uintptr_t)k & 15) == 0;
+    const dim3 grid((dv + 31) / 32, H, n_seq);
+    if (dk <= 4 * DR_LPR) launch_delta<4>(p, grid, vec, ST(stream));
+    else if (dk <= 8 * DR_LPR) launch_delta<8>(p, grid, vec, ST(stream));
+    else if (dk <= 16 * DR_LPR) launch_delta<16>(p, grid, vec, ST(stream));
+    else launch_delta<32>(p, grid, vec, ST(stream));
     MI355_LAUNCH_CHECK("delta_rule_ragged");
     return 0;
 }
@@ -417,8 +553,39 @@ __global__ __launch_bounds__(256) void glu_rows_kernel(int64_t R, int F, const v
     }
 }
 
+__global__ __launch_bounds__(256) void glu_rows_vec_kernel(int64_t R, int F, const void* __restrict__ in, int in_dt, int64_t ldi, int kind, float limit, void* __restrict__ out,
+                                                           int out_dt, int64_t ldo) {
+    const int F4 = F / 4;
+    const int64_t total = R * F4;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = e / F4;
+        const int i = 4 * (int)(e % F4);
+        const f32x4 g4 = ld4_dt(in, in_dt, r * ldi + i), u4 = ld4_dt(in, in_dt, r * ldi + F + i);
+        f32x4 o;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float g = g4[q], u = u4[q];
+            if (kind == 0) {
+                o[q] = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+            } else {
+                g = fminf(g, limit);
+                u = fminf(fmaxf(u, -limit), limit);
+                o[q] = g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+            }
+        }
+        st4_dt(out, out_dt, r * ldo + i, o);
+    }
+}
+
 extern "C" int mi355_glu_rows(int64_t rows, int F, const void* in, int in_dt, int64_t ld_in, int kind, float limit, void* out, int out_dt, int64_t ld_out, void* stream) {
     MI355_REQUIRE(rows > 0 && F > 0 && in && out && rec_dt_ok(in_dt) && rec_dt_ok(out_dt) && ld_in >= 2 * (int64_t)F && ld_out >= F && (kind == 0 || kind == 1), "glu_rows: bad arguments");
+    if (F % 4 == 0 && ld_in % 4 == 0 && ld_out % 4 == 0 && al16(in) && al16(out)) {
+        const int64_t total4 = rows * (F / 4);
+        const int g4 = (int)((total4 + 255) / 256 > 65535 * 8 ? 65535 * 8 : (total4 + 255) / 256);
+        glu_rows_vec_kernel<<<g4, 256, 0, ST(stream)>>>(rows, F, in, in_dt, ld_in, kind, limit, out, out_dt, ld_out);
+        MI355_LAUNCH_CHECK("glu_rows");
+        return 0;
+    }
     const int64_t total = rows * F;
     const int g = (int)((total + 255) / 256 > 65535 * 8 ? 65535 * 8 : (total + 255) / 256);
     glu_rows_kernel<<<g, 256, 0, ST(stream)>>>(rows, F, in, in_dt, ld_in, kind, limit, out, out_dt, ld_out);

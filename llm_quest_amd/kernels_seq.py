@@ -357,8 +357,9 @@ def delta_rule(q, k, v, b, a, A_log, dt_bias, qscale, seq_off, slot, state, H, G
         if t.dtype != F32 or t.numel() != H or not t.is_contiguous():
             raise ValueError("delta_rule: A_log and dt_bias fp32 [H]")
     o = torch.empty((T, H * dv), dtype=F32, device=q.device)
-    L.call("mi355_delta_rule_ragged", n_seq, L.ptr(seq_off), L.ptr(slot), H, G, dk, dv, L.ptr(q), L.ptr(k), _dt(q), q.stride(0), k.stride(0), L.ptr(v), _dt(v), v.stride(0),
-           L.ptr(b), L.ptr(a), _dt(b), b.stride(0), a.stride(0), L.ptr(A_log), L.ptr(dt_bias), float(qscale), L.ptr(state), L.ptr(o))
+    ws = torch.empty((T * H * 4,), dtype=F32, device=q.device)  # per token and head: decay, beta, the two unit-vector factors
+    L.call("mi355_delta_rule_ragged", T, n_seq, L.ptr(seq_off), L.ptr(slot), H, G, dk, dv, L.ptr(q), L.ptr(k), _dt(q), q.stride(0), k.stride(0), L.ptr(v), _dt(v), v.stride(0),
+           L.ptr(b), L.ptr(a), _dt(b), b.stride(0), a.stride(0), L.ptr(A_log), L.ptr(dt_bias), float(qscale), L.ptr(state), L.ptr(o), L.ptr(ws))
     return o
 
 

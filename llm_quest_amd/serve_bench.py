@@ -1,6 +1,6 @@
 """Serving throughput of the registry models with random weights: prompts (one packed step) and one-token steps through the slot cache, beside the
 closest existing model of the package at equal width and depth -- the Qwen3.5 hybrid text stack (gated delta net + gated attention, dense SwiGLU) through
-its own cache.  ``bench.py --serve gemepel`` prints the result as one JSON line; the default workload of ``bench.py`` is untouched.
+its own cache.  ``bench.py --serve gemepel`` (or ``--serve mepatar``) prints the result as one JSON line; the default workload of ``bench.py`` is untouched.
 
 Sizes resemble real layers (random weights; what is generated means nothing): width 1024 / 2048, 4 layers (three linear-attention layers and one softmax-
 attention layer, as the Qwen3.5 stack has them), 16 experts of which 2 run per token."""
@@ -42,6 +42,38 @@ def random_gemepel(width, heads, device, decay_rank=64):
     return model
 
 
+def mepatar_config(width, heads, vocab=32000):
+    """Two gated-delta-rule layers, one retention layer and one sliding-window attention layer (512 keys + 4 kept), 16 heads x 128 x 128 in the recurrent
+    mixers; three layers with 16 experts (2 per token, ff = 1.75 width) and one dense layer (ff = 3.5 width); 4 taps, norms in 2 groups."""
+    rec = {"heads": 16, "dim": 128, "vdim": 128}
+    ret = dict(rec, decay=[1.0 - 2.0 ** (-5 - 0.25 * i) for i in range(16)], rot={"dims": 128, "base": 1e6})
+    dlt = dict(rec, kv_heads=16, conv=4)
+    att = {"heads": heads, "kv_heads": 2, "dim": 128, "vdim": 128, "mask": {"size": 512, "keep_first": 4}, "rot": {"dims": 64, "base": 1e6}, "scale": 128 ** -0.5}
+    moe = {"kind": "moe", "expert": {"ff": int(width * 1.75), "limit": 7.0}, "router": {"experts": 16, "top": 2}}
+    dense = {"kind": "dense", "ff": int(width * 3.5)}
+    layers = [{"type": "delta", "mixer": dlt, "mlp": moe}, {"type": "retention", "mixer": ret, "mlp": dense}, {"type": "delta", "mixer": dlt, "mlp": moe},
+              {"type": "attention", "mixer": att, "mlp": moe}]
+    return {"architecture": "Mepatar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6, "groups": 2}, "canon": {"taps": 4}, "embedding": {"scale": 1.0}, "layers": layers}
+
+
+def random_mepatar(width, heads, device):
+    from llm_quest_amd.mepatar.mepatar_model import MepatarConfig, MepatarModel
+
+    with torch.device(device):
+        model = MepatarModel(MepatarConfig(mepatar_config(width, heads)))
+    g = torch.Generator(device=device).manual_seed(7)
+    for name, p in model.named_parameters():
+        if name.endswith("canon.weight") or name.endswith("mixer.conv"):
+            p.data.copy_((0.3 * torch.randn(p.shape, device=device, generator=g)).to(BF16))
+        elif p.dim() >= 2:
+            p.data.copy_((torch.randn(p.shape, device=device, generator=g) / p.shape[-1] ** 0.5).to(BF16))
+        elif "norm" in name or name.endswith("temp"):
+            p.data.fill_(1.0)
+        elif name.endswith("A_log"):
+            p.data.fill_(-2.0)
+    return model
+
+
 def _time(fn, warmup, steps):
     for _ in range(warmup):
         fn()
@@ -54,9 +86,16 @@ def _time(fn, warmup, steps):
 
 
 def bench_gemepel(width, heads, batch, prompt, steps, warmup, device):
+    return bench_ragged(random_gemepel(width, heads, device), f"gemepel-w{width}", batch, prompt, steps, warmup)
+
+
+def bench_mepatar(width, heads, batch, prompt, steps, warmup, device):
+    return bench_ragged(random_mepatar(width, heads, device), f"mepatar-w{width}", batch, prompt, steps, warmup)
+
+
+def bench_ragged(model, name, batch, prompt, steps, warmup):
     from llm_quest_amd.generate import RaggedBatch
 
-    model = random_gemepel(width, heads, device)
     vocab = model.vocab_size
     g = torch.Generator().manual_seed(1)
     prompts = [torch.randint(0, vocab, (prompt,), generator=g).tolist() for _ in range(batch)]
@@ -86,7 +125,7 @@ def bench_gemepel(width, heads, batch, prompt, steps, warmup, device):
     rb.step([("solo", prompts[0])])
     t_solo = _time(lambda: rb.step([("solo", [5])]), warmup, steps)
     params = sum(p.numel() for p in model.parameters())
-    return {"model": f"gemepel-w{width}", "params_M": round(params / 1e6, 1), "prefill_tok_s": round(batch * prompt / t_prefill), "prefill_ms": round(t_prefill * 1e3, 2),
+    return {"model": name, "params_M": round(params / 1e6, 1), "prefill_tok_s": round(batch * prompt / t_prefill), "prefill_ms": round(t_prefill * 1e3, 2),
             "decode_tok_s": round(batch / t_decode), "decode_ms_per_step": round(t_decode * 1e3, 3), "decode_b1_ms_per_step": round(t_solo * 1e3, 3)}
 
 
@@ -133,11 +172,12 @@ def bench_qwen35(width, heads, batch, prompt, steps, warmup, device):
 
 
 def run(which, steps, warmup, sizes=((1024, 8), (2048, 16)), batch=8, prompt=1024, device="cuda", with_reference=True):
-    if which != "gemepel":
-        raise SystemExit(f"--serve: unknown model {which!r}")
+    benches = {"gemepel": bench_gemepel, "mepatar": bench_mepatar}
+    if which not in benches:
+        raise SystemExit(f"--serve: unknown model {which!r} (known: {sorted(benches)})")
     rows = []
     for width, heads in sizes:
-        rows.append(bench_gemepel(width, heads, batch, prompt, steps, warmup, device))
+        rows.append(benches[which](width, heads, batch, prompt, steps, warmup, device))
         if with_reference:
             rows.append(bench_qwen35(width, heads, batch, prompt, steps, warmup, device))
     out = {"metric": "serving throughput (random weights)", "unit": "tokens/s", "batch": batch, "prompt": prompt, "steps": steps, "warmup": warmup,
