@@ -414,6 +414,8 @@ int mi355_pad_tokens(int B, int L, const int64_t* flat_ids, const int64_t* offse
  * stream, one wave per output column.  bf16 in / out, fp32 accumulate. */
 int mi355_gemv_bf16(int M, int64_t N, int K, const void* x, int64_t ldx, const void* W, int64_t ldw, void* y, int64_t ldy, const void* residual,
                     int64_t ldr, void* stream);
+/* The same weight stream with fp32 results: y fp32 [M, N] = x W^T (+ bias fp32 [N], may be NULL). */
+int mi355_gemv_bf16_f32out(int M, int64_t N, int K, const void* x, int64_t ldx, const void* W, int64_t ldw, float* y, int64_t ldy, const float* bias, void* stream);
 /* The same weight stream with the row operation that feeds it folded in -- a one-token step is bound by its launch count (12 -> 6 per
  * block): prologue 1 = x rows are RMS-normalised with weight norm_w / eps first (PytorchRMSNorm, qwen3_attention.py:19-29, in front of the QKV,
  * gate-up and head projections); prologue 2 = x holds the fused lin1 | lin_gate rows [M, 2K] and the operand is lin1 * silu(lin_gate)
@@ -531,11 +533,11 @@ int mi355_rope_heads(int64_t tokens, int H, int n, const void* src, int src_dt, 
 int mi355_gated_headnorm(int64_t tokens, int H, int D, const float* o, const float* w, const void* gate, int g_dt, int64_t ldg, float eps, void* out,
                          int out_dt, int64_t ldo, void* stream);
 /* Gated linear attention over the rows [seq_off[s], seq_off[s+1]) of each sequence s, state[slot[s]] (fp32 [H, dk, dv]) read and written:
- * S <- diag(a_t) S + k_t v_t^T, o_t = S^T (q_t * qscale), a_t = sigmoid(z_t + zbias)^inv_tau.  q / k rows [H * dk], v rows [H * dv] of dtype dt, z rows [H * dk] of dtype z_dt,
+ * S <- diag(a_t) S + k_t v_t^T, o_t = S^T (q_t * qscale), a_t = sigmoid(z_t + zbias)^inv_tau.  q / k rows [H * dk] of dtype dt, v rows [H * dv] of dtype v_dt, z rows [H * dk] of dtype z_dt,
  * o fp32 [tokens, H * dv].  dk <= 256.  head_decay (fp32 [H], may be NULL): if given, a_t = head_decay[h] for every key channel of head h (retention with a
  * fixed decay per head; z and zbias may then be NULL).  k_t is multiplied by kscale before it enters the state. */
 int mi355_gla_fwd(int n_seq, const int* seq_off, const int* slot, int H, int dk, int dv, const void* q, const void* k, const void* v, const void* z, int dt,
-                  int z_dt, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldz, const float* zbias, float inv_tau, float qscale, const float* head_decay,
+                  int z_dt, int v_dt, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldz, const float* zbias, float inv_tau, float qscale, const float* head_decay,
                   float kscale, float* state, float* o, void* stream);
 /* logits[t, e] = sum_k x[t, k] W[e, k]: fp32 rows (pitch ldx) against a bf16 matrix [E, K] (pitch ldw), fp32 FMA; out fp32 [tokens, E]. */
 int mi355_router_logits(int64_t tokens, int E, int K, const float* x, int64_t ldx, const void* W, int64_t ldw, float* out, void* stream);

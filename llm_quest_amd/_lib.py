@@ -93,6 +93,7 @@ SIGNATURES = {
     "mi355_pad_tokens": [_I, _I, _P, _P, _L, _P, _P, _P],
     # KV-cache decoding (csrc/decode.hip)
     "mi355_gemv_bf16": [_I, _L, _I, _P, _L, _P, _L, _P, _L, _P, _L, _P],
+    "mi355_gemv_bf16_f32out": [_I, _L, _I, _P, _L, _P, _L, _P, _L, _P, _P],
     "mi355_gemv_bf16_pro": [_I, _L, _I, _P, _L, _I, _P, _F, _P, _L, _P, _L, _P, _L, _P],
     "mi355_attn_decode_qkv": [_I, _I, _I, _I, _P, _L, _P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _P, _P, _P, _L, _P, _F, _F, _I, _P, _P],
     "mi355_decode_advance": [_I, _P, _P, _P, _P, _P, _P],
@@ -107,7 +108,7 @@ SIGNATURES = {
     "mi355_latent_kv_append": [_L, _I, _I, _P, _I, _L, _P, _F, _P, _P, _P, _I, _P, _I, _L, _P],
     "mi355_rope_heads": [_L, _I, _I, _P, _I, _L, _I, _I, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P],
     "mi355_gated_headnorm": [_L, _I, _I, _P, _P, _P, _I, _L, _F, _P, _I, _L, _P],
-    "mi355_gla_fwd": [_I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _I, _L, _L, _L, _L, _P, _F, _F, _P, _F, _P, _P, _P],
+    "mi355_gla_fwd": [_I, _P, _P, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _L, _L, _L, _L, _P, _F, _F, _P, _F, _P, _P, _P],
     "mi355_router_logits": [_L, _I, _I, _P, _L, _P, _L, _P, _P],
     "mi355_moe_route": [_L, _I, _I, _I, _I, _P, _P, _F, _I, _P, _P, _P],
     "mi355_moe_dispatch": [_L, _I, _P, _P, _P, _P],

@@ -56,6 +56,37 @@ __global__ __launch_bounds__(256) void gemv_kernel(int M, int64_t N, int K, cons
     }
 }
 
+// The same weight stream with fp32 results (+ an fp32 bias per column): rows whose consumer works in fp32 (rotary, norms, gates of a recurrence).
+template <int MT>
+__global__ __launch_bounds__(256) void gemv_f32out_kernel(int M, int64_t N, int K, const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ W,
+                                                          int64_t ldw, float* __restrict__ y, int64_t ldy, const float* __restrict__ bias) {
+    const int lane = threadIdx.x & 63;
+    const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    const bf16_t* w = W + n * ldw;
+    float acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m] = 0.f;
+    for (int k0 = lane * 8; k0 < K; k0 += 512) {
+        float wf[8];
+        unpack8(*reinterpret_cast<const u32x4*>(w + k0), wf);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            if (m >= M) break;
+            float xf[8];
+            unpack8(*reinterpret_cast<const u32x4*>(x + m * ldx + k0), xf);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[m] = fmaf(wf[e], xf[e], acc[m]);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        if (m >= M) break;
+        const float s = wave_sum(acc[m]);
+        if (lane == 0) y[m * ldy + n] = bias ? s + bias[n] : s;
+    }
+}
+
 __device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
     u32x4 o;
 #pragma unroll
@@ -517,6 +548,19 @@ extern "C" int mi355_gemv_bf16(int M, int64_t N, int K, const void* x, int64_t l
     if (M == 1) LAUNCH(1); else if (M == 2) LAUNCH(2); else if (M <= 4) LAUNCH(4); else LAUNCH(8);
 #undef LAUNCH
     MI355_LAUNCH_CHECK("gemv_bf16");
+    return 0;
+}
+
+extern "C" int mi355_gemv_bf16_f32out(int M, int64_t N, int K, const void* x, int64_t ldx, const void* W, int64_t ldw, float* y, int64_t ldy, const float* bias,
+                                      void* stream) {
+    MI355_REQUIRE(M >= 1 && M <= 8, "gemv_bf16_f32out: 1..8 rows (got %d)", M);
+    MI355_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K && ldy >= N, "gemv_bf16_f32out: K and the leading dimensions of x / W must be multiples of 8");
+    MI355_REQUIRE(x && W && y, "gemv_bf16_f32out: null pointer");
+    const int grid = (int)((N + 3) / 4);
+#define LAUNCH(MT) gemv_f32out_kernel<MT><<<grid, 256, 0, ST(stream)>>>(M, N, K, (const bf16_t*)x, ldx, (const bf16_t*)W, ldw, y, ldy, bias)
+    if (M == 1) LAUNCH(1); else if (M == 2) LAUNCH(2); else if (M <= 4) LAUNCH(4); else LAUNCH(8);
+#undef LAUNCH
+    MI355_LAUNCH_CHECK("gemv_bf16_f32out");
     return 0;
 }
 

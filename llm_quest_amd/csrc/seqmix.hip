@@ -356,7 +356,7 @@ extern "C" int mi355_gated_headnorm(int64_t tokens, int H, int D, const float* o
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
 __global__ void gla_kernel(const int* __restrict__ seq_off, const int* __restrict__ slot, int H, int dk, int dv, const void* __restrict__ q, const void* __restrict__ k,
-                           const void* __restrict__ v, const void* __restrict__ z, int dt, int z_dt, int64_t ldq, int64_t ldk, int64_t ldv_, int64_t ldz,
+                           const void* __restrict__ v, const void* __restrict__ z, int dt, int z_dt, int v_dt, int64_t ldq, int64_t ldk, int64_t ldv_, int64_t ldz,
                            const float* __restrict__ zbias, float inv_tau, float qscale, const float* __restrict__ head_decay, float kscale,
                            float* __restrict__ state, float* __restrict__ o) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -399,7 +399,7 @@ __global__ void gla_kernel(const int* __restrict__ seq_off, const int* __restric
             rv[u] = 0.f;
             if (e < nt * 64) {
                 const int j = e >> 6, c = blockIdx.z * 64 + (e & 63);
-                if (c < dv) rv[u] = ld_dt(v, dt, (int64_t)(tb + j) * ldv_ + (int64_t)h * dv + c);
+                if (c < dv) rv[u] = ld_dt(v, v_dt, (int64_t)(tb + j) * ldv_ + (int64_t)h * dv + c);
             }
         }
     };
@@ -469,16 +469,16 @@ __global__ void gla_kernel(const int* __restrict__ seq_off, const int* __restric
 }
 
 extern "C" int mi355_gla_fwd(int n_seq, const int* seq_off, const int* slot, int H, int dk, int dv, const void* q, const void* k, const void* v, const void* z, int dt,
-                             int z_dt, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldz, const float* zbias, float inv_tau, float qscale, const float* head_decay, float kscale,
+                             int z_dt, int v_dt, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldz, const float* zbias, float inv_tau, float qscale, const float* head_decay, float kscale,
                              float* state, float* o, void* stream) {
-    MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && seq_off && slot && H > 0 && H <= 65535 && dk > 0 && dk <= 16 * GLA_R && dv > 0 && q && k && v && state && o && dt_ok(dt),
+    MI355_REQUIRE(n_seq > 0 && n_seq <= 65535 && seq_off && slot && H > 0 && H <= 65535 && dk > 0 && dk <= 16 * GLA_R && dv > 0 && q && k && v && state && o && dt_ok(dt) && dt_ok(v_dt),
                   "gla_fwd: bad arguments (key channels per head <= 256)");
     MI355_REQUIRE(head_decay || (z && zbias && dt_ok(z_dt) && ldz >= (int64_t)H * dk), "gla_fwd: the decay needs its rows and bias, or a constant per head");
     MI355_REQUIRE(ldq >= (int64_t)H * dk && ldk >= (int64_t)H * dk && ldv >= (int64_t)H * dv, "gla_fwd: rows too short");
     const int RC = (dk + GLA_R - 1) / GLA_R;
     const size_t lds_bytes = sizeof(float) * ((size_t)3 * GLA_TB * dk + (size_t)GLA_TB * 64 + (size_t)GLA_TB * RC * 64);
     MI355_REQUIRE(lds_bytes <= 64 * 1024, "gla_fwd: LDS budget exceeded");
-    gla_kernel<<<dim3(n_seq, H, (dv + 63) / 64), 64 * RC, lds_bytes, ST(stream)>>>(seq_off, slot, H, dk, dv, q, k, v, z, dt, z_dt, ldq, ldk, ldv, ldz, zbias, inv_tau, qscale,
+    gla_kernel<<<dim3(n_seq, H, (dv + 63) / 64), 64 * RC, lds_bytes, ST(stream)>>>(seq_off, slot, H, dk, dv, q, k, v, z, dt, z_dt, v_dt, ldq, ldk, ldv, ldz, zbias, inv_tau, qscale,
                                                                                    head_decay, kscale, state, o);
     MI355_LAUNCH_CHECK("gla_fwd");
     return 0;

@@ -139,7 +139,7 @@ def gla(q, k, v, z, zbias, inv_tau, qscale, seq_off, slot, state, H, dk, dv, hea
     if state.dtype != F32 or not state.is_contiguous() or tuple(state.shape[1:]) != (H, dk, dv) or zbias.dtype != F32 or zbias.numel() != H * dk:
         raise ValueError("gla: state fp32 [slots, H, dk, dv], bias fp32 [H * dk]")
     o = torch.empty((q.shape[0], H * dv), dtype=F32, device=q.device)
-    L.call("mi355_gla_fwd", n_seq, L.ptr(seq_off), L.ptr(slot), H, dk, dv, L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(z), _dt(q), _dt(z), q.stride(0), k.stride(0), v.stride(0),
+    L.call("mi355_gla_fwd", n_seq, L.ptr(seq_off), L.ptr(slot), H, dk, dv, L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(z), _dt(q), _dt(z), _dt(v), q.stride(0), k.stride(0), v.stride(0),
            z.stride(0), L.ptr(zbias), float(inv_tau), float(qscale), None, float(kscale), L.ptr(state), L.ptr(o))
     return o
 
@@ -147,15 +147,15 @@ def gla(q, k, v, z, zbias, inv_tau, qscale, seq_off, slot, state, H, dk, dv, hea
 def _gla_fixed(q, k, v, head_decay, qscale, kscale, seq_off, slot, state, H, dk, dv):
     for t, n, w in ((q, "q", H * dk), (k, "k", H * dk), (v, "v", H * dv)):
         _rows(t, f"gla({n})")
-        if t.shape[1] != w or t.dtype != q.dtype or t.shape[0] != q.shape[0]:
-            raise ValueError(f"gla({n}): [tokens, {w}] of q's dtype required")
+        if t.shape[1] != w or (n != "v" and t.dtype != q.dtype) or t.shape[0] != q.shape[0]:
+            raise ValueError(f"gla({n}): [tokens, {w}] required (k of q's dtype)")
     n_seq = slot.numel()
     _i32(seq_off, "gla(seq_off)", n_seq + 1)
     _i32(slot, "gla(slot)")
     if state.dtype != F32 or not state.is_contiguous() or tuple(state.shape[1:]) != (H, dk, dv):
         raise ValueError("gla: state fp32 [slots, H, dk, dv]")
     o = torch.empty((q.shape[0], H * dv), dtype=F32, device=q.device)
-    L.call("mi355_gla_fwd", n_seq, L.ptr(seq_off), L.ptr(slot), H, dk, dv, L.ptr(q), L.ptr(k), L.ptr(v), None, _dt(q), 0, q.stride(0), k.stride(0), v.stride(0),
+    L.call("mi355_gla_fwd", n_seq, L.ptr(seq_off), L.ptr(slot), H, dk, dv, L.ptr(q), L.ptr(k), L.ptr(v), None, _dt(q), 0, _dt(v), q.stride(0), k.stride(0), v.stride(0),
            0, None, 1.0, float(qscale), L.ptr(head_decay), float(kscale), L.ptr(state), L.ptr(o))
     return o
 
@@ -222,6 +222,11 @@ def linear(x, w, out_dtype=None, bias=None):
             from . import ops_decode
 
             return ops_decode.gemv(x, w)
+        if aligned and M <= 8 and out_dtype == F32 and (bias is None or (bias.dtype == F32 and bias.is_contiguous() and bias.numel() == N)):
+            L.require_gpu(x, w, bias)
+            out = torch.empty((M, N), dtype=F32, device=x.device)
+            L.call("mi355_gemv_bf16_f32out", M, N, Kd, L.ptr(x), x.stride(0), L.ptr(w), w.stride(0), L.ptr(out), out.stride(0), L.ptr(bias))
+            return out
         if aligned and M > 8:
             return K.gemm(L.GEMM_NT, x, w, out_dtype=out_dtype, bias=bias)
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
