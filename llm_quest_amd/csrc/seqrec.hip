@@ -230,7 +230,9 @@ __global__ __launch_bounds__(256) void ragged_conv_kernel(int64_t T, int C, int 
     }
 }
 
-// Four channels per thread, one token per blockIdx.x (C % 4 == 0, 16-byte aligned rows).
+// Four channels per thread, one token per blockIdx.x (C % 4 == 0, 16-byte aligned rows).  TAPS > 0: the thread's 4 x TAPS weights are TAPS consecutive
+// 16-byte words (w is [C, TAPS] and the channel a multiple of 4), fetched as such; TAPS == 0: any number of taps, one weight at a time.
+template <int TAPS>
 __global__ __launch_bounds__(256) void ragged_conv_vec_kernel(int C, int taps, const void* __restrict__ x, int x_dt, int64_t ldx, const float* __restrict__ w,
                                                               const int* __restrict__ row_seq, const int* __restrict__ seq_off, const int* __restrict__ slot,
                                                               const float* __restrict__ state, int act, int residual, void* __restrict__ y, int y_dt, int64_t ldy) {
@@ -242,12 +244,30 @@ __global__ __launch_bounds__(256) void ragged_conv_vec_kernel(int C, int taps, c
     const int local = (int)(t - start);
     const float* st = state + (int64_t)slot[s] * (taps - 1) * C;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f}, cur = {0.f, 0.f, 0.f, 0.f};
-    for (int j = 0; j < taps; ++j) {
-        const int sl = local - (taps - 1) + j;
-        const f32x4 in = sl >= 0 ? ld4_dt(x, x_dt, (int64_t)(start + sl) * ldx + c) : *(const f32x4*)(st + (int64_t)(taps - 1 + sl) * C + c);
-        if (j == taps - 1) cur = in;
+    if constexpr (TAPS > 0) {
+        float wf[4 * TAPS];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] = fmaf(w[(c + e) * taps + j], in[e], acc[e]);
+        for (int i = 0; i < TAPS; ++i) {
+            const f32x4 wv = *(const f32x4*)(w + (int64_t)c * TAPS + 4 * i);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) wf[4 * i + e] = wv[e];
+        }
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {
+            const int sl = local - (TAPS - 1) + j;
+            const f32x4 in = sl >= 0 ? ld4_dt(x, x_dt, (int64_t)(start + sl) * ldx + c) : *(const f32x4*)(st + (int64_t)(TAPS - 1 + sl) * C + c);
+            if (j == TAPS - 1) cur = in;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = fmaf(wf[e * TAPS + j], in[e], acc[e]);
+        }
+    } else {
+        for (int j = 0; j < taps; ++j) {
+            const int sl = local - (taps - 1) + j;
+            const f32x4 in = sl >= 0 ? ld4_dt(x, x_dt, (int64_t)(start + sl) * ldx + c) : *(const f32x4*)(st + (int64_t)(taps - 1 + sl) * C + c);
+            if (j == taps - 1) cur = in;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = fmaf(w[(c + e) * taps + j], in[e], acc[e]);
+        }
     }
     if (act == 1) {
 #pragma unroll
@@ -286,7 +306,17 @@ extern "C" int mi355_ragged_conv(int64_t tokens, int n_seq, int C, int taps, con
     MI355_REQUIRE(rec_dt_ok(x_dt) && rec_dt_ok(y_dt) && ldx >= C && ldy >= C && (act == 0 || act == 1), "ragged_conv: bad operands");
     const int64_t total = tokens * C;
     if (C % 4 == 0 && ldx % 4 == 0 && ldy % 4 == 0 && al16(x) && al16(y) && al16(state) && tokens < ((int64_t)1 << 31)) {
-        ragged_conv_vec_kernel<<<dim3((unsigned)tokens, (C / 4 + 255) / 256), 256, 0, ST(stream)>>>(C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy);
+        const dim3 grid((unsigned)tokens, (C / 4 + 255) / 256);
+#define CONV_CASE(TP)                                                                                                                                          \
+    case TP:                                                                                                                                                   \
+        ragged_conv_vec_kernel<TP><<<grid, 256, 0, ST(stream)>>>(C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy);      \
+        break;
+        switch (al16(w) ? taps : 0) {
+            CONV_CASE(2) CONV_CASE(3) CONV_CASE(4) CONV_CASE(5) CONV_CASE(6) CONV_CASE(7) CONV_CASE(8)
+            default:
+                ragged_conv_vec_kernel<0><<<grid, 256, 0, ST(stream)>>>(C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy);
+        }
+#undef CONV_CASE
     } else {
         const int g = (int)((total + 255) / 256 > 65535 * 8 ? 65535 * 8 : (total + 255) / 256);
         ragged_conv_kernel<<<g, 256, 0, ST(stream)>>>(tokens, C, taps, x, x_dt, ldx, w, row_seq, seq_off, slot, state, act, residual, y, y_dt, ldy);
