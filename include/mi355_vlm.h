@@ -552,10 +552,12 @@ int mi355_moe_dispatch(int64_t entries, int E, const int* ids, int* offs, int* p
 /* C[b][m, n] = epi(sum_k A[b][m, k] B[b][n, k]) with general strides: A at b * a_bs + row * lda + k, B at b * b_bs + n * sbn + k * sbk (one of sbn / sbk
  * is 1), C at b * c_bs + row * ldc + n.  grp_offs (may be NULL): batch b owns the sorted rows [grp_offs[b], grp_offs[b+1]) and M bounds their number;
  * a_rows: sorted row r reads A row a_rows[r] / a_div; c_rows: it writes C row c_rows[r]; row_scale: that C row is scaled.  epi 1 = relu(x)^2.
- * use_mfma needs bf16 A and B; otherwise fp32 FMA accumulation in a fixed k order.  bias (fp32 [N], may be NULL) is added to every row before epi. */
+ * use_mfma needs bf16 A and B; otherwise fp32 FMA accumulation in a fixed k order.  bias (fp32 [N], may be NULL) is added to every row before epi.
+ * epi 2 / 3 (gated feed-forward): B's rows come in blocks of 64 = [32 gate rows | 32 up rows] (N a multiple of 64), C has n_out <= N / 2 columns,
+ * C[m, 32 b + i] = act(gate, up) of block b: 2 = g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit); 3 = gelu_tanh(gate) * up. */
 int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t lda, int64_t a_bs, const void* B, int b_dt, int64_t sbn, int64_t sbk,
                 int64_t b_bs, void* C, int c_dt, int64_t ldc, int64_t c_bs, const int* grp_offs, const int* a_rows, int a_div, const int* c_rows,
-                const float* row_scale, int epi, int use_mfma, const float* bias, void* stream);
+                const float* row_scale, int epi, int use_mfma, const float* bias, float limit, int n_out, void* stream);
 /* Causal attention with two-part keys over ragged batches: sequence s has n_new[s] query rows starting at row q_row0[s], `past[s]` earlier keys;
  * key j of it is K1 row k1_row0[s] + j (head stride k1_hs, D1 wide), K2 row k2_row0[s] + j (shared by heads, D2 wide), value row v_row0[s] + j.
  * Q fp32 [.., H, D1 + D2]; K1 / K2 / V / O of dtype dt.  A tile covers 32 / hm tokens x hm heads (hm > 1 needs k1_hs == v_hs == 0); the MFMA path (bf16,

@@ -112,7 +112,7 @@ SIGNATURES = {
     "mi355_router_logits": [_L, _I, _I, _P, _L, _P, _L, _P, _P],
     "mi355_moe_route": [_L, _I, _I, _I, _I, _P, _P, _F, _I, _P, _P, _P],
     "mi355_moe_dispatch": [_L, _I, _P, _P, _P, _P],
-    "mi355_bgemm": [_I, _I, _I, _I, _P, _I, _L, _L, _P, _I, _L, _L, _L, _P, _I, _L, _L, _P, _P, _I, _P, _P, _I, _I, _P, _P],
+    "mi355_bgemm": [_I, _I, _I, _I, _P, _I, _L, _L, _P, _I, _L, _L, _L, _P, _I, _L, _L, _P, _P, _I, _P, _P, _I, _I, _P, _F, _I, _P],
     "mi355_latent_attn": [_I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _F, _I, _I, _P, _L, _I, _I, _I, _P],
     # parallel-sublayer hybrid decoders in ragged batches (csrc/seqrec.hip)
     "mi355_group_rmsnorm_sum": [_L, _I, _P, _P, _I, _L, _P, _I, _L, _I, _P, _I, _F, _P, _P, _I, _P, _P, _P, _I, _P, _P],

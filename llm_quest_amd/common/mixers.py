@@ -416,8 +416,13 @@ class SoftmaxTopkMoE(_Frozen):
         super().__init__()
         self.width, self.ff, self.experts, self.top, self.limit = width, ff, experts, top, float(limit)
         self.w_router = self._param(experts, width)
-        self.w_gate_up = self._param(experts, 2 * ff, width)
+        self.w_gate_up = self._param(experts, 64 * (-(-ff // 32)), width)  # per expert S.pack_gate_up(gate, up): [32 gate rows | 32 up rows] blocks
         self.w_down = self._param(experts, width, ff)
+
+    def load_experts(self, gates, ups, downs):
+        """Per-expert weight lists in the checkpoint's layout ([ff, width], [ff, width], [width, ff]) -> the stacked parameters."""
+        self.w_gate_up.data.copy_(torch.stack([S.pack_gate_up(g, u) for g, u in zip(gates, ups)]))
+        self.w_down.data.copy_(torch.stack(list(downs)))
 
     @torch.no_grad()
     def step(self, h32, h):
@@ -426,9 +431,10 @@ class SoftmaxTopkMoE(_Frozen):
         logits = S.router_logits(h32, self.w_router)
         ids, wts = S.moe_route(logits, None, top, 1, 1, 1.0, softmax=True)
         offs, perm = S.moe_dispatch(ids.view(-1), E)
-        gu = torch.empty((T * top, 2 * ff), dtype=h.dtype, device=h.device)
-        S.bgemm(h, self.w_gate_up, gu, T * top, 2 * ff, self.width, batch=E, sbn=self.width, b_bs=2 * ff * self.width, grp_offs=offs, a_rows=perm, a_div=top)
-        act = S.glu_rows(gu, S.GLU_CLAMPED_SWISH, self.limit)
+        np_ = self.w_gate_up.shape[1]
+        act = torch.empty((T * top, ff), dtype=h.dtype, device=h.device)  # the gated activation is the gate-up product's epilogue
+        S.bgemm(h, self.w_gate_up, act, T * top, np_, self.width, batch=E, sbn=self.width, b_bs=np_ * self.width, grp_offs=offs, a_rows=perm, a_div=top,
+                epi=S.EPI_CLAMPED_SWISH_GLU, limit=self.limit, n_out=ff)
         out = torch.empty((T * top, self.width), dtype=F32, device=h.device)
         S.bgemm(act, self.w_down, out, T * top, self.width, ff, batch=E, sbn=ff, b_bs=self.width * ff, grp_offs=offs, c_rows=perm, row_scale=wts.view(-1))
         return out

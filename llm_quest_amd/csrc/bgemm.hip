@@ -31,9 +31,22 @@ struct BgemmArgs {
     const int* c_rows;       // or null: sorted row r writes C row c_rows[r]
     const float* row_scale;  // or null: C row (after c_rows) is multiplied by row_scale[that row]
     const float* bias;       // or null: bias[n] is added to column n before the epilogue
-    int epi;                 // 0 none, 1 relu(x)^2
+    int epi;                 // 0 none, 1 relu(x)^2, 2 / 3 gated (see gated_act): B's rows come in blocks of 64 = [32 gate rows | 32 up rows], C has n_out columns
+    float limit;
+    int n_out;
     int a_dt, b_dt, c_dt;
 };
+
+// Gated activations of a feed-forward's [gate | up] product.  2: g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1).
+// 3: gelu_tanh(gate) * up.
+__device__ __forceinline__ float gated_act(int epi, float g, float u, float limit) {
+    if (epi == 2) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+    }
+    return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+}
 
 __device__ __forceinline__ float ldx(const void* p, int dt, int64_t i) { return dt == MI355_DT_F32 ? ((const float*)p)[i] : bf2f(((const bf16_t*)p)[i]); }
 
@@ -90,7 +103,7 @@ __global__ __launch_bounds__(256) void bgemm_fma_kernel(BgemmArgs p) {
         for (int k = 0; k < BK; ++k) {
             float a[4], bb[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i], bb[i] = Bs[k][tx * 4 + i];
+            for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i], bb[i] = Bs[k][(i >> 1) * 32 + tx * 2 + (i & 1)];  // columns 2 tx, 2 tx + 1 and the same + 32: a gate and its up
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -106,9 +119,20 @@ __global__ __launch_bounds__(256) void bgemm_fma_kernel(BgemmArgs p) {
         const int64_t crow = p.c_rows ? p.c_rows[r] : r;
         const float sc = p.row_scale ? p.row_scale[crow] : 1.0f;
         const int64_t cb = (int64_t)b * p.c_bs + crow * p.ldc;
+        if (p.epi >= 2) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int n = (n0 >> 1) + tx * 2 + j;  // gate column n0 + 2 tx + j, up column 32 further
+                if (n >= p.n_out) continue;
+                const float v = gated_act(p.epi, acc[i][j], acc[i][j + 2], p.limit) * sc;
+                if (p.c_dt == MI355_DT_F32) ((float*)p.C)[cb + n] = v;
+                else ((bf16_t*)p.C)[cb + n] = f2bf(v);
+            }
+            continue;
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int n = n0 + tx * 4 + j;
+            const int n = n0 + (j >> 1) * 32 + tx * 2 + (j & 1);
             if (n >= p.N) continue;
             float v = acc[i][j] + (p.bias ? p.bias[n] : 0.f);
             if (p.epi == 1) v = v > 0.f ? v * v : 0.f;
@@ -307,6 +331,15 @@ __global__ __launch_bounds__(256) void bgemm_mfma128_kernel(BgemmArgs p) {
                 const int64_t crow = p.c_rows ? p.c_rows[r] : r;
                 const float sc = p.row_scale ? p.row_scale[crow] : 1.0f;
                 const int64_t cb = (int64_t)b * p.c_bs + crow * p.ldc;
+                if (p.epi >= 2) {  // this wave's 64 columns are one [32 gates | 32 ups] block: the lane holds a gate (bj = 0) and its up (bj = 1)
+                    const int n = ((n0 + wn) >> 1) + ln;
+                    if (n < p.n_out) {
+                        const float v = gated_act(p.epi, acc[bi][0][4 * g + i], acc[bi][1][4 * g + i], p.limit) * sc;
+                        if (p.c_dt == MI355_DT_F32) ((float*)p.C)[cb + n] = v;
+                        else ((bf16_t*)p.C)[cb + n] = f2bf(v);
+                    }
+                    continue;
+                }
 #pragma unroll
                 for (int bj = 0; bj < 2; ++bj) {
                     const int n = n0 + wn + 32 * bj + ln;
@@ -322,11 +355,12 @@ __global__ __launch_bounds__(256) void bgemm_mfma128_kernel(BgemmArgs p) {
 
 extern "C" int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_dt, int64_t lda, int64_t a_bs, const void* B, int b_dt, int64_t sbn, int64_t sbk,
                            int64_t b_bs, void* C, int c_dt, int64_t ldc, int64_t c_bs, const int* grp_offs, const int* a_rows, int a_div, const int* c_rows,
-                           const float* row_scale, int epi, int use_mfma, const float* bias, void* stream) {
+                           const float* row_scale, int epi, int use_mfma, const float* bias, float limit, int n_out, void* stream) {
     MI355_REQUIRE(batch > 0 && batch <= 65535 && M > 0 && N > 0 && K > 0 && A && B && C, "bgemm: bad arguments");
     MI355_REQUIRE((a_dt == MI355_DT_BF16 || a_dt == MI355_DT_F32) && (b_dt == MI355_DT_BF16 || b_dt == MI355_DT_F32) && (c_dt == MI355_DT_BF16 || c_dt == MI355_DT_F32),
                   "bgemm: bad dtype");
-    MI355_REQUIRE(epi == 0 || epi == 1, "bgemm: bad epilogue");
+    MI355_REQUIRE(epi >= 0 && epi <= 3, "bgemm: bad epilogue");
+    MI355_REQUIRE(epi < 2 || (N % 64 == 0 && n_out > 0 && n_out <= N / 2 && !bias), "bgemm: a gated epilogue takes B rows in [32 gate | 32 up] blocks (N a multiple of 64), n_out <= N / 2 columns, no bias");
     MI355_REQUIRE(!a_rows || a_div >= 1, "bgemm: gathered rows need a divisor >= 1");
     MI355_REQUIRE(sbn >= 1 && sbk >= 1 && (sbn == 1 || sbk == 1), "bgemm: one of B's strides must be 1");
     MI355_REQUIRE(!use_mfma || (a_dt == MI355_DT_BF16 && b_dt == MI355_DT_BF16), "bgemm: the MFMA path takes bf16 operands");
@@ -336,8 +370,9 @@ extern "C" int mi355_bgemm(int batch, int M, int N, int K, const void* A, int a_
     p.M = M, p.N = N, p.K = K;
     p.grp_offs = grp_offs, p.a_rows = a_rows, p.a_div = a_rows ? a_div : 1, p.c_rows = c_rows, p.row_scale = row_scale;
     p.bias = bias;
+    p.limit = limit, p.n_out = n_out;
     p.epi = epi, p.a_dt = a_dt, p.b_dt = b_dt, p.c_dt = c_dt;
-    if (use_mfma && sbk == 1 && N >= 128 && K >= 64) {  // the large tile: weights stored [out, in], enough columns to fill it
+    if (use_mfma && ((sbk == 1 && N >= 128 && K >= 64) || epi >= 2)) {  // (a gated epilogue needs a gate and its up in one lane: this kernel's 64 columns per wave)  // the large tile: weights stored [out, in], enough columns to fill it
         const int64_t my128 = ((int64_t)M + TM - 1) / TM;
         MI355_REQUIRE(my128 <= 65535, "bgemm: too many row tiles");
         bgemm_mfma128_kernel<<<dim3((N + TM - 1) / TM, (unsigned)my128, batch), 256, 0, ST(stream)>>>(p);

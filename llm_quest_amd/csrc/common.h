@@ -43,27 +43,6 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// ---- sums over aligned groups of lanes on DPP (no LDS traffic)
-template <int CTRL>
-__device__ __forceinline__ float dpp_f(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
-template <int W>
-__device__ __forceinline__ float lanes_sum(float v) {  // all-reduce over aligned groups of W (4, 8 or 16) lanes
-    static_assert(W == 4 || W == 8 || W == 16, "lanes_sum: 4, 8 or 16");
-    if constexpr (W == 16) {
-        v += dpp_f<0x128>(v);  // row_ror:8
-        v += dpp_f<0x124>(v);  // row_ror:4
-        v += dpp_f<0x122>(v);  // row_ror:2
-        v += dpp_f<0x121>(v);  // row_ror:1
-    } else {
-        v += dpp_f<0xB1>(v);  // quad_perm:[1,0,3,2]
-        v += dpp_f<0x4E>(v);  // quad_perm:[2,3,0,1]
-        if constexpr (W == 8) v += dpp_f<0x141>(v);  // row_half_mirror: the other quad of the 8-lane group
-    }
-    return v;
-}
-
 // ---- SwiGLU: one definition for the elementwise kernels and the GEMM epilogues, so fused == separate bit for bit.  sigmoid through v_exp + v_rcp
 // (1 ulp each; an IEEE division costs ten instructions per element, and the epilogues are bound by what their lanes issue); operands and results
 // are rounded to bf16 where the reference's bf16 tensors are (silu(g) is a bf16 tensor before it multiplies u, qwen3_transformer_block.py:48-53).

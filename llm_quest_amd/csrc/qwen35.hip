@@ -14,6 +14,7 @@
 //   gated_rmsnorm        RMSNorm(fp32) * silu(gate) -> bf16
 //   rowmask              x * padding_mask
 #include "common.h"
+#include "lane_sums.h"
 
 namespace {
 
@@ -39,6 +40,7 @@ __device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
 }
 // Cross-lane sums on the VALU (DPP / permlane swaps), not through the LDS crossbar: ds_bpermute (what __shfl_xor compiles to)
 // costs an LDS round trip per step of every reduction, and the recurrence kernels below are one dependent chain per time step.
+// (dpp_f / lanes_sum: lane_sums.h.)
 // v[lane] + v[lane ^ 16] + v[lane ^ 32] + v[lane ^ 48]: the same element of the wave's four 16-lane rows
 __device__ __forceinline__ float rows_sum(float v) {
     auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);

@@ -6,6 +6,7 @@
 // Conventions as in seqmix.hip: operands come as bf16 or fp32 (a MI355_DT_* code each); the residual stream, norm statistics, rotary angles, decays,
 // gates of a recurrence and recurrent state are fp32 in both modes.  A "row" is a token of the packed batch; sequences are described by int32 device arrays.
 #include "common.h"
+#include "lane_sums.h"
 
 #define ST(s) ((hipStream_t)(s))
 

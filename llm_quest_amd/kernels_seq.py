@@ -194,7 +194,7 @@ def moe_dispatch(ids, E):
 
 
 def bgemm(a, b, c, M, N, Kd, batch=1, lda=None, a_bs=0, sbn=None, sbk=1, b_bs=0, ldc=None, c_bs=0, grp_offs=None, a_rows=None, a_div=1, c_rows=None,
-          row_scale=None, epi=0, mfma=None, bias=None):
+          row_scale=None, epi=0, mfma=None, bias=None, limit=0.0, n_out=0):
     """The general strided product (see include/mi355_vlm.h).  Strides default to a's / c's row pitch and b stored [N, K]; the caller vouches that the
     strides stay inside the tensors.  ``mfma`` defaults to bf16 a and b."""
     L.require_gpu(a, b, c, grp_offs, a_rows, c_rows, row_scale, bias)
@@ -203,7 +203,7 @@ def bgemm(a, b, c, M, N, Kd, batch=1, lda=None, a_bs=0, sbn=None, sbk=1, b_bs=0,
     if mfma is None:
         mfma = a.dtype == BF16 and b.dtype == BF16
     L.call("mi355_bgemm", batch, M, N, Kd, L.ptr(a), _dt(a), a.stride(0) if lda is None else lda, a_bs, L.ptr(b), _dt(b), b.stride(0) if sbn is None else sbn, sbk, b_bs,
-           L.ptr(c), _dt(c), c.stride(0) if ldc is None else ldc, c_bs, L.ptr(grp_offs), L.ptr(a_rows), a_div, L.ptr(c_rows), L.ptr(row_scale), epi, 1 if mfma else 0, L.ptr(bias))
+           L.ptr(c), _dt(c), c.stride(0) if ldc is None else ldc, c_bs, L.ptr(grp_offs), L.ptr(a_rows), a_div, L.ptr(c_rows), L.ptr(row_scale), epi, 1 if mfma else 0, L.ptr(bias), float(limit), int(n_out))
     return c
 
 
@@ -369,6 +369,21 @@ def delta_rule(q, k, v, b, a, A_log, dt_bias, qscale, seq_off, slot, state, H, G
 
 
 GLU_GELU_TANH, GLU_CLAMPED_SWISH = 0, 1
+EPI_RELU2, EPI_CLAMPED_SWISH_GLU, EPI_GELU_TANH_GLU = 1, 2, 3  # epilogues of bgemm
+
+
+def pack_gate_up(gate, up):
+    """[F, K] gate and up weights -> [64 * ceil(F / 32), K]: blocks of 32 gate rows followed by their 32 up rows (zero rows pad the last block), the
+    layout the gated epilogues of ``bgemm`` read -- a lane of the product then holds a gate and its up."""
+    F, Kd = gate.shape
+    nb = -(-F // 32)
+    out = gate.new_zeros((nb, 2, 32, Kd))
+    pad = nb * 32 - F
+    g = torch.cat([gate, gate.new_zeros((pad, Kd))]) if pad else gate
+    u = torch.cat([up, up.new_zeros((pad, Kd))]) if pad else up
+    out[:, 0] = g.reshape(nb, 32, Kd)
+    out[:, 1] = u.reshape(nb, 32, Kd)
+    return out.reshape(nb * 64, Kd)
 
 
 def glu_rows(x, kind, limit=0.0, out_dtype=None):

@@ -3,7 +3,8 @@
 Tensor names of the checkpoint: ``embed``, ``head``, ``final.norm``, and per layer i ``l<i>.norm1|norm2``, ``l<i>.canon1`` (the input convolution),
 ``l<i>.mix.*`` (retention: q, k, v, g, o; attention: q, k, v, o each with ``.b``, q.norm, k.norm, temp; delta: q, k, v each with ``.conv``, b, a, A_log,
 dt_bias, norm, g, o) and ``l<i>.mlp.*`` (dense: gate, up, down; experts: router, e<j>.gate, e<j>.up, e<j>.down).  Projections that share their input are
-stored side by side in one parameter, the experts of a layer stacked in one, so that each group is one product.
+stored side by side in one parameter, the experts of a layer stacked in one (gate and up rows in alternating blocks of 32, so that the gated activation is
+the product's epilogue), so that each group is one product.
 """
 
 import json
@@ -61,6 +62,6 @@ def load_mepatar_state(model, w):
             _put(blk.ff.w_down, w[e + "down"])
         else:
             _put(blk.ff.w_router, w[e + "router"])
-            blk.ff.w_gate_up.data.copy_(torch.stack([torch.cat([w[f"{e}e{j}.gate"], w[f"{e}e{j}.up"]], dim=0) for j in range(blk.ff.experts)]))
-            blk.ff.w_down.data.copy_(torch.stack([w[f"{e}e{j}.down"] for j in range(blk.ff.experts)]))
+            n = range(blk.ff.experts)
+            blk.ff.load_experts([w[f"{e}e{j}.gate"] for j in n], [w[f"{e}e{j}.up"] for j in n], [w[f"{e}e{j}.down"] for j in n])
     return model

@@ -113,7 +113,10 @@ def test_config_reader_and_loader_fuse_the_projections(tmp_path):
     assert torch.equal(b0.mixer.w_in, torch.cat([w["l0.mix.q"], w["l0.mix.k"], w["l0.mix.v"], w["l0.mix.g"]]))
     assert torch.equal(b1.mixer.w_qkv, torch.cat([w["l1.mix.q"], w["l1.mix.k"], w["l1.mix.v"]])) and torch.equal(b1.mixer.b_qkv, torch.cat([w["l1.mix.q.b"], w["l1.mix.k.b"], w["l1.mix.v.b"]]))
     assert torch.equal(b2.mixer.w_in, torch.cat([w["l2.mix." + n] for n in "qkvgba"])) and torch.equal(b2.mixer.conv, torch.cat([w["l2.mix." + n + ".conv"] for n in "qkv"]))
-    assert torch.equal(b0.ff.w_gate_up[5], torch.cat([w["l0.mlp.e5.gate"], w["l0.mlp.e5.up"]])) and torch.equal(b1.ff.w_gate_up, torch.cat([w["l1.mlp.gate"], w["l1.mlp.up"]]))
+    gu = b0.ff.w_gate_up[5]  # 40 rows of gate and up each -> two blocks of [32 gate | 32 up], the second one padded with zero rows
+    assert gu.shape[0] == 128 and torch.equal(gu[:32], w["l0.mlp.e5.gate"][:32]) and torch.equal(gu[32:64], w["l0.mlp.e5.up"][:32])
+    assert torch.equal(gu[64:72], w["l0.mlp.e5.gate"][32:]) and torch.equal(gu[96:104], w["l0.mlp.e5.up"][32:]) and float(gu[72:96].abs().max()) == 0 and float(gu[104:].abs().max()) == 0
+    assert torch.equal(b1.ff.w_gate_up, torch.cat([w["l1.mlp.gate"], w["l1.mlp.up"]]))
     assert b3.ff is None and torch.equal(b0.canon.weight, w["l0.canon1"])
     bad = json.loads(json.dumps(cfg))
     bad["layers"][0]["type"] = "convolution"

@@ -477,8 +477,7 @@ def test_mixture_of_experts_alone(dt):
     w = U.make_weights(cfg, 3)
     m = SoftmaxTopkMoE(W, ff, E, top, 0.8)
     m.w_router.data.copy_(w["l0.mlp.router"])
-    m.w_gate_up.data.copy_(torch.stack([torch.cat([w[f"l0.mlp.e{j}.gate"], w[f"l0.mlp.e{j}.up"]]) for j in range(E)]))
-    m.w_down.data.copy_(torch.stack([w[f"l0.mlp.e{j}.down"] for j in range(E)]))
+    m.load_experts([w[f"l0.mlp.e{j}.gate"] for j in range(E)], [w[f"l0.mlp.e{j}.up"] for j in range(E)], [w[f"l0.mlp.e{j}.down"] for j in range(E)])
     m = m.to(DEV)
     h = torch.randn(T, W, generator=g)
     act = F32 if dt == "float32" else BF16
