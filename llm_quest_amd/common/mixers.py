@@ -3,7 +3,12 @@
 * ``LatentAttention``       -- multi-head latent attention: queries and keys / values go through low-rank latents, one rotated key part is shared by all
   heads, only the normalised latent and that rotated part are cached (optionally another layer's);
 * ``GatedLinearAttention``  -- linear attention with a per-key-channel decay and a matrix state per head, carried in fp32;
-* ``GroupedSigmoidMoE``     -- sigmoid-scored experts chosen inside the best groups, squared-ReLU experts.
+* ``GroupedSigmoidMoE``     -- sigmoid-scored experts chosen inside the best groups, squared-ReLU experts;
+* ``ShortConvInput``        -- h + conv(h), a short causal convolution over time in front of a mixer, its last inputs carried per sequence;
+* ``Retention``             -- linear attention with one fixed decay per head (rotate-half rotary, gated unit-RMS output);
+* ``SlidingWindowAttention``-- grouped-query softmax attention with biases, query / key norm, a temperature per head and a window that keeps the first tokens;
+* ``GatedDeltaRule``        -- the gated delta rule behind short convolutions, unit-vector queries and keys, a matrix state per value head in fp32;
+* ``GatedMLP`` / ``SoftmaxTopkMoE`` -- a dense GELU-gated layer; softmax-routed experts with a clamped gated activation, weights = the winners' scores.
 
 They run one *step* of a batch (``SeqStep``): the new tokens of every sequence, packed row after row, against what ``utils.SlotStateCache`` holds.  Inference
 only, HIP kernels only (``kernels_seq``); weights are bf16, what is normalised, rotated, decayed, accumulated over time or routed is fp32.

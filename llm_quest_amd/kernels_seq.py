@@ -1,6 +1,7 @@
-"""Python launchers of the ragged-batch serving kernels (csrc/seqmix.hip, csrc/bgemm.hip, csrc/latent_attn.hip): hashed-bigram embedding,
-post-sum LayerNorm on an fp32 residual stream, latent key/value rows, interleaved rotary embedding, two-part-key attention, gated linear
-attention with carried state, the grouped sigmoid router and the grouped expert products.
+"""Python launchers of the ragged-batch serving kernels (csrc/seqmix.hip, csrc/bgemm.hip, csrc/latent_attn.hip, csrc/seqrec.hip): hashed-bigram embedding,
+post-sum LayerNorm on an fp32 residual stream, latent key/value rows, rotary embedding in both pair layouts, two-part-key / grouped-query / windowed attention,
+gated linear attention and retention with carried state, the sigmoid and softmax routers and the grouped expert products (with gated epilogues), the residual
+sum with RMS norms in groups, short convolutions with carried inputs, query / key / value rows into a slot cache, the gated delta rule, gated activations.
 
 Activations are bf16 (serving mode: bf16 operands, fp32 accumulation) or fp32 (true 32-bit mode: every product is an fp32 FMA chain; the bf16
 weights are exactly representable and widened on load).  Whatever the mode, the residual stream, norm statistics, rotary angles, decays,
