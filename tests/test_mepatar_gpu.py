@@ -490,3 +490,35 @@ def test_mixture_of_experts_alone(dt):
         for e, a in zip(ids[t].tolist(), wts[t]):
             want[t] += a * O.expert_ff(hq[t : t + 1].double(), wd, f"l0.mlp.e{e}.", 0.8)[0]
     assert row_err(out, want) < (1e-5 if dt == "float32" else 2e-2)
+
+
+def test_trace_replay_program_end_to_end(checkpoint, tmp_path):
+    """bin/trace_run as a user runs it: a folder, steps on standard input (two prompts in one batch, then one token each, one request ending early and
+    its slot taken by a third), logits files out -- against the oracle."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    folder, cfg, w = checkpoint
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    a, b, c = tokens(31, cfg["vocab"], 50), tokens(9, cfg["vocab"], 51), tokens(12, cfg["vocab"], 52)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:28], "want": [0, 13, 27]}, {"id": "b", "tokens": b[:8], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[28:29], "want": [0]}, {"id": "b", "tokens": b[8:9], "want": [0]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[29:30], "want": []}], "end": []},
+             {"step": 3, "entries": [{"id": "c", "tokens": c, "want": [11]}], "end": ["c"]},
+             {"step": 4, "entries": [{"id": "a", "tokens": a[30:31], "want": [0]}], "end": ["a"]}]
+    wa, wb, wc = oracle(cfg, w, a), oracle(cfg, w, b), oracle(cfg, w, c)
+    want = {0: torch.stack([wa[0], wa[13], wa[27]]), 1: torch.stack([wa[28], wb[8]]), 3: wc[11:12], 4: wa[30:31]}
+    for dt in ("float32", "bfloat16"):
+        out = tmp_path / dt
+        res = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dt, "--out", str(out), "--max-tokens", "64"],
+                             input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+        assert res.returncode == 0, res.stderr[-2000:]
+        assert [l for l in res.stdout.split("\n") if l.startswith("done")] == [f"done {i}" for i in range(5)]
+        assert not (out / "2.f32").exists()
+        for i, ref in want.items():
+            got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, cfg["vocab"]))
+            assert got.shape == ref.shape and model_err(got, ref, dt) < TOL[dt], (dt, i)
