@@ -258,7 +258,8 @@ def latent_attn(q, k1, k2, v, out, H, hm, D1, D2, DV, q_hs, k1_hs, v_hs, o_hs, d
         _i32(t, "latent_attn(desc)", n_seq)
     mfma = v.dtype == BF16
     splits, ws = 1, None
-    if mfma and D1 + D2 <= 320 and DV <= 256 and max_keys and not window:
+    # (a window that can hide keys leaves a one-token step window + keep_first visible keys, and the kernel skips the others 64 at a time: nothing to deal out)
+    if mfma and D1 + D2 <= 320 and DV <= 256 and max_keys and (not window or window >= max_keys):
         head_tiles = -(-H // hm)
         splits = attn_key_splits(n_seq, head_tiles, max_new, hm, max_keys)
         if splits > 1:

@@ -522,3 +522,10 @@ def test_trace_replay_program_end_to_end(checkpoint, tmp_path):
         for i, ref in want.items():
             got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, cfg["vocab"]))
             assert got.shape == ref.shape and model_err(got, ref, dt) < TOL[dt], (dt, i)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_one_token_step_over_a_long_cache_under_a_window_that_hides_nothing(dt):
+    """2 000 cached keys and a window wider than that: the bf16 kernel deals the keys to several workgroups; a hot key far back must come through."""
+    got, want = _attention_case(dt, 6, 3, 32, 48, 4000, 5, 2000, 1, [37])
+    assert want[0, 0, 0] > 30 and row_err(got.reshape(1, -1), want.reshape(1, -1)) < (2e-5 if dt == "float32" else 2e-2)
