@@ -44,7 +44,7 @@ def random_gemepel(width, heads, device, decay_rank=64):
 
 def mepatar_config(width, heads, vocab=32000):
     """Two gated-delta-rule layers, one retention layer and one sliding-window attention layer (512 keys + 4 kept), 16 heads x 128 x 128 in the recurrent
-    mixers; three layers with 16 experts (2 per token, ff = 1.75 width) and one dense layer (ff = 3.5 width); 4 taps, norms in 2 groups."""
+    mixers; three layers with 16 experts (2 per token, ff = 1.75 width) and one dense layer (ff = 3.5 width); 4 taps, norms in 4 groups."""
     rec = {"heads": 16, "dim": 128, "vdim": 128}
     ret = dict(rec, decay=[1.0 - 2.0 ** (-5 - 0.25 * i) for i in range(16)], rot={"dims": 128, "base": 1e6})
     dlt = dict(rec, kv_heads=16, conv=4)
@@ -53,7 +53,7 @@ def mepatar_config(width, heads, vocab=32000):
     dense = {"kind": "dense", "ff": int(width * 3.5)}
     layers = [{"type": "delta", "mixer": dlt, "mlp": moe}, {"type": "retention", "mixer": ret, "mlp": dense}, {"type": "delta", "mixer": dlt, "mlp": moe},
               {"type": "attention", "mixer": att, "mlp": moe}]
-    return {"architecture": "Mepatar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6, "groups": 2}, "canon": {"taps": 4}, "embedding": {"scale": 1.0}, "layers": layers}
+    return {"architecture": "Mepatar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6, "groups": 4}, "canon": {"taps": 4}, "embedding": {"scale": 1.0}, "layers": layers}
 
 
 def random_mepatar(width, heads, device):
